@@ -1,0 +1,189 @@
+/*
+ * smat.h -- C ABI of the MI355X (gfx950) block-sparse SpMM library.
+ *
+ *     C (M x N) = A (M x K, 16x16 blocked CSR, fp16) * B (K x N, dense fp16),
+ *     fp32 accumulation on the fp16 MFMA units.
+ *
+ * Everything here is `extern "C"`, takes plain pointers and sizes, and returns
+ * an int status (SMAT_OK == 0).  A host compiled with g++ needs no HIP header:
+ * device memory, streams and events are reachable through the thin wrappers at
+ * the end of this file.  Citations name the file:line of the reference
+ * (spcl/smat) interface that each entry point replaces.
+ */
+#ifndef SMAT_H
+#define SMAT_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define SMAT_BS 16 /* block edge: MMA_M == MMA_K, src/cuda_hgemm/src/common/matrix.h:13-15 */
+
+/* ---- status ------------------------------------------------------------- */
+#define SMAT_OK 0
+#define SMAT_ERR_INVALID (-1)     /* bad argument (shape not a multiple of 16/8, NULL, ...) */
+#define SMAT_ERR_HIP (-2)         /* a HIP runtime call failed; see smat_last_error()       */
+#define SMAT_ERR_NOMEM (-3)       /* host or device allocation failed                       */
+#define SMAT_ERR_IO (-4)          /* file could not be opened / parsed                      */
+#define SMAT_ERR_UNSUPPORTED (-5) /* valid request this build does not implement            */
+
+/* Text of the most recent error on the calling thread ("" if none). */
+const char *smat_last_error(void);
+/* "smat-amd <version> gfx950" */
+const char *smat_version(void);
+
+/* ---- SpMM: the drop-in entry point --------------------------------------
+ * Replaces `void mmaCBTKernel(half *bcsrValuesA, int *bcsrRowPtrA,
+ * int *bcsrColIdxA, half *B, half *C, size_t M, size_t N, size_t K,
+ * size_t nonzeroBlocks, int *blockInfo, int *relativeBlockIndexMapping)`
+ * (src/cuda_hgemm/src/mma/mmaCBT.cu:83-88; shape HGEMM_FUNC_SPARSE2,
+ * src/cuda_hgemm/src/main.cu:7) -- same positional arguments, same meaning:
+ *
+ *   vals     device, fp16, nnzb*256, block p at vals[p*256], row-major in block
+ *   row_ptr  device, int32, M/16+1
+ *   col_idx  device, int32, nnzb, ABSOLUTE first column of each block (matrix.h:455)
+ *   B        device, fp16, column-major K x N: element (k,n) at B[n*K+k] (mmaCBT.cu:52)
+ *   C        device, fp16, row-major M x N, OVERWRITTEN (mmaCBT.cu:36,72-79)
+ *   M, K     multiples of 16 (mmio_highlevel.h:609-616); N a multiple of 8 (tester.h:40)
+ *   block_info, rel_map   accepted for signature compatibility and ignored: the
+ *            running block index equals the row_ptr/col_idx position
+ *            (matrix.h:425-431 vs 441-463), so the dense maps carry nothing.
+ *
+ * Asynchronous on the null stream like the reference launch; returns a status
+ * where the reference returns void. */
+int smat_spmm_bcsr_f16(const uint16_t *vals, const int32_t *row_ptr, const int32_t *col_idx,
+                       const uint16_t *B, uint16_t *C, size_t M, size_t N, size_t K, size_t nnzb,
+                       const int32_t *block_info, const int32_t *rel_map);
+
+/* ---- SpMM with options / explicit stream / plan -------------------------- */
+#define SMAT_B_COL_MAJOR 0 /* B[n*K + k]: the reference layout               */
+#define SMAT_C_F16 0       /* the reference output type                      */
+#define SMAT_C_F32 1       /* keep the fp32 accumulators                     */
+
+#define SMAT_KERNEL_AUTO 0
+#define SMAT_KERNEL_ROWWISE 1 /* one wavefront per (block-row chunk, N panel), operands straight from L2 */
+#define SMAT_KERNEL_SWEEP 2   /* workgroup sweeps K for a group of block rows, B panel staged in LDS      */
+
+typedef struct smat_spmm_opts {
+    int32_t b_layout; /* SMAT_B_COL_MAJOR                                   */
+    int32_t c_dtype;  /* SMAT_C_F16 | SMAT_C_F32                            */
+    int32_t kernel;   /* SMAT_KERNEL_*                                      */
+    int32_t reserved; /* must be 0                                          */
+    void *stream;     /* hipStream_t, NULL = null stream                    */
+} smat_spmm_opts;
+
+/* A plan is the per-matrix work list (load balancing over block rows of skewed
+ * length).  It plays the role the reference gives to the one-off host-side
+ * BCSR build (SparseMatrix ctor, matrix.h:173): made once per matrix, outside
+ * the timed loop (tester.h:342-358), reused by every launch. */
+typedef struct smat_plan smat_plan;
+
+/* row_ptr_host: the HOST copy of the BCSR row pointer (M/16+1 entries).
+ * col_idx_host: HOST copy of the BCSR column index (may be NULL unless
+ *               opts->kernel requests SMAT_KERNEL_SWEEP).
+ * n_hint: the N the plan will mostly be used with (panel width choice). */
+int smat_plan_create(smat_plan **plan, const int32_t *row_ptr_host, const int32_t *col_idx_host,
+                     size_t M, size_t K, size_t nnzb, size_t n_hint, const smat_spmm_opts *opts);
+int smat_plan_destroy(smat_plan *plan);
+/* Fills info[0..7]: kernel id, work items, split block rows, chunk size,
+ * workspace bytes, panel width, 0, 0. */
+int smat_plan_info(const smat_plan *plan, int64_t *info);
+
+/* Same operands as smat_spmm_bcsr_f16; C is uint16_t* or float* per opts->c_dtype.
+ * opts == NULL means defaults; plan == NULL means no work list (whole block
+ * rows, one wavefront each). */
+int smat_spmm_bcsr_f16_ex(const uint16_t *vals, const int32_t *row_ptr, const int32_t *col_idx,
+                          const uint16_t *B, void *C, size_t M, size_t N, size_t K, size_t nnzb,
+                          const smat_spmm_opts *opts, const smat_plan *plan);
+
+/* ---- matrix load: Matrix Market -> CSR (host) ----------------------------
+ * Replaces mmio_allinone (src/cuda_hgemm/src/common/mmio_highlevel.h:619-786):
+ * M and K come back rounded up to multiples of 16, symmetric/hermitian files
+ * are mirrored, entries keep file order inside a row, duplicates are kept,
+ * values go double -> fp16.  Returns SMAT_OK or SMAT_ERR_IO; *ref_code receives
+ * the reference's own code (-1 open, -2 banner, -4 size line; may be NULL).
+ * Arrays are allocated by the library: release with smat_host_free. */
+int smat_mtx_read(const char *path, size_t *M, size_t *K, size_t *nnz, int *is_symmetric,
+                  int32_t **row_ptr, int32_t **col_idx, uint16_t **val, int *ref_code);
+void smat_host_free(void *p);
+
+/* ---- blocking: CSR -> 16x16 BCSR (host) -----------------------------------
+ * Replaces SparseMatrix::csrToBcsr (src/cuda_hgemm/src/common/matrix.h:376-502)
+ * and emits bit-identical row_ptr / col_idx / val without the two dense
+ * (M/16)x(K/16) maps.  counts[0..2] = nonzero, "dense", "sparse" blocks as the
+ * reference logs them (matrix.h:176, 2:4 heuristic matrix.h:400-419).
+ * block_info / rel_map: pass non-NULL pointers only if the dense maps are
+ * really wanted (they are (M/16)*(K/16) ints each); NULL skips them. */
+int smat_csr_to_bcsr(size_t M, size_t K, const int32_t *row_ptr, const int32_t *col_idx,
+                     const uint16_t *val, int64_t *counts, int32_t **b_row_ptr,
+                     int32_t **b_col_idx, uint16_t **b_val, int32_t **block_info,
+                     int32_t **rel_map);
+
+/* ---- reorder (host) --------------------------------------------------------
+ * Row clustering that minimises the number of nonzero blocks: the reference's
+ * `Matrix_Blocking -a 5 -F 1` path, BlockingEngine::GetGrouping
+ * (preprocess/src/general/blocking.cpp:616-657) -> IterativeBlockingKeeper
+ * (blocking.cpp:431-547) with JaccardDistanceGroup (blocking.cpp:904-975),
+ * merge_rows (preprocess/src/general/utilities.cpp:145-173) and
+ * get_fixed_size_grouping / get_permutation (utilities.cpp:8-54).
+ *
+ *   rows, row_ptr (int64, rows+1), col_idx (int64, sorted ascending in a row)
+ *   col_block / row_block / tau : the -b / -B / -t flags (input.h:88-105)
+ *   grouping  out, int64[rows]: block-row id of each row (the ".g" GROUPING line)
+ *   perm      out, int64[rows]: perm[new_row] = old_row (CSR::reorder, csr.cpp:97-105)
+ *   stats     out, int64[4]: comparison_counter, merge_counter,
+ *             VBR_nzblocks_count, VBR_longest_row (utilities.cpp:217-224,
+ *             blocking.cpp:562-614); may be NULL
+ */
+int smat_reorder_rows(int64_t rows, int64_t cols, const int64_t *row_ptr, const int64_t *col_idx,
+                      int64_t col_block, int64_t row_block, float tau, int64_t *grouping,
+                      int64_t *perm, int64_t *stats);
+
+/* Row pass, then the same pass on the transpose of the row-permuted pattern
+ * (what src/reorder.py:107-139,143-182 does through files), on a CSR with
+ * int32 indices.  Trailing empty rows/columns keep their place, as they do not
+ * exist in the reference's edge-list files (csr.cpp:262-263).
+ * perm_rows[new]=old (M entries), perm_cols[new]=old (K entries). */
+int smat_reorder_csr(size_t M, size_t K, const int32_t *row_ptr, const int32_t *col_idx,
+                     int64_t col_block, int64_t row_block, float tau, int do_cols,
+                     int64_t *perm_rows, int64_t *perm_cols, int64_t *stats_rows,
+                     int64_t *stats_cols);
+
+/* Applies perm_rows / perm_cols (either may be NULL = identity) to a CSR with
+ * values; columns inside a row come out ascending.  Output arrays are
+ * allocated by the library (smat_host_free). */
+int smat_permute_csr(size_t M, size_t K, const int32_t *row_ptr, const int32_t *col_idx,
+                     const uint16_t *val, const int64_t *perm_rows, const int64_t *perm_cols,
+                     int32_t **out_row_ptr, int32_t **out_col_idx, uint16_t **out_val);
+
+/* ---- thin device runtime wrappers (so hosts need no HIP headers) ----------
+ * Stand in for the cudaMalloc / cudaMemcpy / cudaMemset / cudaDeviceSynchronize
+ * calls of Matrix / SparseMatrix (matrix.h:30,40,78-101,158-199) and for
+ * CudaTimer (src/cuda_hgemm/src/common/cuda_timer.h:7-45). */
+int smat_device_count(int *n);
+int smat_set_device(int dev);
+int smat_device_name(int dev, char *buf, size_t len);
+int smat_device_attr(int dev, int64_t *cus, int64_t *lds_bytes, int64_t *mem_bytes, int64_t *clock_khz);
+int smat_malloc(void **dptr, size_t bytes);
+int smat_free(void *dptr);
+int smat_memcpy_h2d(void *dst, const void *src, size_t bytes);
+int smat_memcpy_d2h(void *dst, const void *src, size_t bytes);
+int smat_memcpy_d2d(void *dst, const void *src, size_t bytes);
+int smat_memset(void *dptr, int byte, size_t bytes);
+int smat_device_synchronize(void);
+int smat_stream_create(void **stream);
+int smat_stream_destroy(void *stream);
+int smat_stream_synchronize(void *stream);
+int smat_event_create(void **event);
+int smat_event_destroy(void *event);
+int smat_event_record(void *event, void *stream);
+int smat_event_synchronize(void *event);
+int smat_event_elapsed_ms(void *start, void *stop, float *ms);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* SMAT_H */

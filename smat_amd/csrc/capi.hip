@@ -1,0 +1,268 @@
+// C ABI over the HIP kernels: SpMM entry points, plans (work lists) and the thin
+// runtime wrappers that let a g++-compiled host live without HIP headers.
+// Interface contract: include/smat.h.
+#include <hip/hip_runtime.h>
+
+#include <algorithm>
+#include <cstdarg>
+#include <cstdio>
+#include <cstring>
+#include <new>
+#include <vector>
+
+#include "../../include/smat.h"
+#include "errors.h"
+#include "spmm_kernels.h"
+
+using namespace smat;
+
+#define SMAT_HIP(call)                                                                     \
+    do {                                                                                   \
+        hipError_t e_ = (call);                                                            \
+        if (e_ != hipSuccess)                                                              \
+            return set_error(SMAT_ERR_HIP, "%s failed: %s (%s:%d)", #call,                 \
+                             hipGetErrorString(e_), __FILE__, __LINE__);                   \
+    } while (0)
+
+struct smat_plan {
+    int kernel = SMAT_KERNEL_ROWWISE;
+    size_t M = 0, K = 0, nnzb = 0, n_cap = 0;
+    int chunk = 0;
+    int panel_tiles = 0;
+    int n_items = 0, n_split_rows = 0, n_slots = 0;
+    WorkItem *d_items = nullptr;
+    SplitRow *d_split = nullptr;
+    float *d_workspace = nullptr;
+    size_t workspace_bytes = 0;
+};
+
+extern "C" const char *smat_version(void) { return "smat-amd 0.1 gfx950"; }
+
+static int check_shapes(const void *vals, const void *row_ptr, const void *col_idx, const void *B,
+                        const void *C, size_t M, size_t N, size_t K, size_t nnzb)
+{
+    if (!row_ptr || !B || !C) return set_error(SMAT_ERR_INVALID, "row_ptr, B and C must not be NULL");
+    if (nnzb && (!vals || !col_idx))
+        return set_error(SMAT_ERR_INVALID, "vals and col_idx must not be NULL when nnzb > 0");
+    if (M == 0 || N == 0 || K == 0) return set_error(SMAT_ERR_INVALID, "M, N, K must be positive");
+    if (M % 16 || K % 16)
+        return set_error(SMAT_ERR_INVALID, "M (%zu) and K (%zu) must be multiples of 16", M, K);
+    if (N % 8) return set_error(SMAT_ERR_INVALID, "N (%zu) must be a multiple of 8", N);
+    if (M / 16 > 0x7ffffff0u || N > 0x7ffffff0u || nnzb > 0x7ffffff0u)
+        return set_error(SMAT_ERR_INVALID, "dimension exceeds the int32 index range of BCSR");
+    if ((reinterpret_cast<uintptr_t>(vals) | reinterpret_cast<uintptr_t>(B) |
+         reinterpret_cast<uintptr_t>(C)) & 15)
+        return set_error(SMAT_ERR_INVALID, "vals, B and C must be 16-byte aligned");
+    return SMAT_OK;
+}
+
+extern "C" int smat_spmm_bcsr_f16_ex(const uint16_t *vals, const int32_t *row_ptr,
+                                      const int32_t *col_idx, const uint16_t *B, void *C, size_t M,
+                                      size_t N, size_t K, size_t nnzb, const smat_spmm_opts *opts,
+                                      const smat_plan *plan)
+{
+    int rc = check_shapes(vals, row_ptr, col_idx, B, C, M, N, K, nnzb);
+    if (rc) return rc;
+    smat_spmm_opts o = {SMAT_B_COL_MAJOR, SMAT_C_F16, SMAT_KERNEL_AUTO, 0, nullptr};
+    if (opts) o = *opts;
+    if (o.b_layout != SMAT_B_COL_MAJOR)
+        return set_error(SMAT_ERR_UNSUPPORTED, "only column-major B (B[n*K+k]) is implemented");
+    if (o.c_dtype != SMAT_C_F16 && o.c_dtype != SMAT_C_F32)
+        return set_error(SMAT_ERR_INVALID, "c_dtype must be SMAT_C_F16 or SMAT_C_F32");
+    if (o.c_dtype == SMAT_C_F32 && (reinterpret_cast<uintptr_t>(C) & 15))
+        return set_error(SMAT_ERR_INVALID, "C must be 16-byte aligned");
+
+    SpmmArgs a{};
+    a.vals = vals; a.row_ptr = row_ptr; a.col_idx = col_idx; a.B = B; a.C = C;
+    a.M = M; a.N = N; a.K = K; a.nnzb = nnzb;
+    a.c_f32 = o.c_dtype == SMAT_C_F32;
+    a.n_items = (int)(M / 16);
+    if (plan) {
+        if (plan->M != M || plan->K != K || plan->nnzb != nnzb)
+            return set_error(SMAT_ERR_INVALID, "plan was built for another matrix (M/K/nnzb differ)");
+        if (plan->n_split_rows && N > plan->n_cap)
+            return set_error(SMAT_ERR_INVALID,
+                             "N (%zu) exceeds the plan's workspace width (%zu): rebuild with n_hint >= N",
+                             N, plan->n_cap);
+        a.items = plan->d_items; a.n_items = plan->n_items;
+        a.split_rows = plan->d_split; a.n_split_rows = plan->n_split_rows;
+        a.workspace = plan->d_workspace;
+        a.panel_tiles = plan->panel_tiles;
+    }
+    hipError_t e = launch_rowwise(a, static_cast<hipStream_t>(o.stream));
+    if (e != hipSuccess)
+        return set_error(SMAT_ERR_HIP, "SpMM launch failed: %s", hipGetErrorString(e));
+    return SMAT_OK;
+}
+
+extern "C" int smat_spmm_bcsr_f16(const uint16_t *vals, const int32_t *row_ptr,
+                                   const int32_t *col_idx, const uint16_t *B, uint16_t *C, size_t M,
+                                   size_t N, size_t K, size_t nnzb, const int32_t *block_info,
+                                   const int32_t *rel_map)
+{
+    (void)block_info;
+    (void)rel_map;
+    return smat_spmm_bcsr_f16_ex(vals, row_ptr, col_idx, B, C, M, N, K, nnzb, nullptr, nullptr);
+}
+
+// ---- plans -----------------------------------------------------------------
+
+extern "C" int smat_plan_create(smat_plan **out, const int32_t *row_ptr_host,
+                                 const int32_t *col_idx_host, size_t M, size_t K, size_t nnzb,
+                                 size_t n_hint, const smat_spmm_opts *opts)
+{
+    (void)col_idx_host;
+    if (!out || !row_ptr_host) return set_error(SMAT_ERR_INVALID, "plan and row_ptr_host must not be NULL");
+    if (M == 0 || M % 16 || K % 16) return set_error(SMAT_ERR_INVALID, "M and K must be positive multiples of 16");
+    if (n_hint == 0 || n_hint % 8) return set_error(SMAT_ERR_INVALID, "n_hint must be a positive multiple of 8");
+    const size_t mb = M / 16;
+    if (row_ptr_host[0] != 0 || (size_t)row_ptr_host[mb] != nnzb)
+        return set_error(SMAT_ERR_INVALID, "row_ptr_host[0] must be 0 and row_ptr_host[M/16] == nnzb");
+    for (size_t i = 0; i < mb; i++)
+        if (row_ptr_host[i + 1] < row_ptr_host[i])
+            return set_error(SMAT_ERR_INVALID, "row_ptr_host must be non-decreasing");
+    if (opts && opts->kernel == SMAT_KERNEL_SWEEP)
+        return set_error(SMAT_ERR_UNSUPPORTED, "SMAT_KERNEL_SWEEP is not implemented");
+
+    smat_plan *p = new (std::nothrow) smat_plan();
+    if (!p) return set_error(SMAT_ERR_NOMEM, "out of host memory");
+    p->M = M; p->K = K; p->nnzb = nnzb; p->n_cap = n_hint;
+    p->panel_tiles = rowwise_panel_tiles(n_hint, 0);
+
+    // A block row is split when it is much longer than the average: chunks of
+    // `chunk` blocks (even, so block pairs stay aligned with the MFMA K = 32).
+    size_t nonempty = 0;
+    for (size_t i = 0; i < mb; i++) nonempty += row_ptr_host[i + 1] > row_ptr_host[i];
+    const double avg = nonempty ? (double)nnzb / (double)nonempty : 0.0;
+    long chunk = (long)(4.0 * avg + 0.5);
+    chunk = std::max(chunk, 64L);
+    chunk = (chunk + 1) & ~1L;
+    p->chunk = (int)chunk;
+
+    std::vector<WorkItem> items;
+    std::vector<SplitRow> split;
+    items.reserve(mb + 16);
+    int slot = 0;
+    for (size_t i = 0; i < mb; i++) { // split rows first: they are the longest items
+        const long len = row_ptr_host[i + 1] - row_ptr_host[i];
+        if (len <= chunk) continue;
+        SplitRow sr{(int32_t)i, slot, slot, 0};
+        for (long b = row_ptr_host[i]; b < row_ptr_host[i + 1]; b += chunk) {
+            const long e = std::min<long>(b + chunk, row_ptr_host[i + 1]);
+            items.push_back(WorkItem{(int32_t)i, (int32_t)b, (int32_t)e, slot++});
+        }
+        sr.slot_end = slot;
+        split.push_back(sr);
+    }
+    for (size_t i = 0; i < mb; i++) {
+        const long len = row_ptr_host[i + 1] - row_ptr_host[i];
+        if (len > chunk) continue;
+        items.push_back(WorkItem{(int32_t)i, row_ptr_host[i], row_ptr_host[i + 1], -1});
+    }
+    p->n_items = (int)items.size();
+    p->n_split_rows = (int)split.size();
+    p->n_slots = slot;
+
+    hipError_t e = hipMalloc(&p->d_items, std::max<size_t>(items.size(), 1) * sizeof(WorkItem));
+    if (e == hipSuccess && !items.empty())
+        e = hipMemcpy(p->d_items, items.data(), items.size() * sizeof(WorkItem), hipMemcpyHostToDevice);
+    if (e == hipSuccess && !split.empty()) {
+        e = hipMalloc(&p->d_split, split.size() * sizeof(SplitRow));
+        if (e == hipSuccess)
+            e = hipMemcpy(p->d_split, split.data(), split.size() * sizeof(SplitRow), hipMemcpyHostToDevice);
+        p->workspace_bytes = (size_t)slot * 16 * n_hint * sizeof(float);
+        if (e == hipSuccess) e = hipMalloc(&p->d_workspace, p->workspace_bytes);
+    }
+    if (e != hipSuccess) {
+        smat_plan_destroy(p);
+        return set_error(SMAT_ERR_HIP, "plan allocation failed: %s", hipGetErrorString(e));
+    }
+    *out = p;
+    return SMAT_OK;
+}
+
+extern "C" int smat_plan_destroy(smat_plan *p)
+{
+    if (!p) return SMAT_OK;
+    if (p->d_items) (void)hipFree(p->d_items);
+    if (p->d_split) (void)hipFree(p->d_split);
+    if (p->d_workspace) (void)hipFree(p->d_workspace);
+    delete p;
+    return SMAT_OK;
+}
+
+extern "C" int smat_plan_info(const smat_plan *p, int64_t *info)
+{
+    if (!p || !info) return set_error(SMAT_ERR_INVALID, "plan and info must not be NULL");
+    info[0] = p->kernel; info[1] = p->n_items; info[2] = p->n_split_rows; info[3] = p->chunk;
+    info[4] = (int64_t)p->workspace_bytes; info[5] = 16 * p->panel_tiles; info[6] = 0; info[7] = 0;
+    return SMAT_OK;
+}
+
+// ---- runtime wrappers --------------------------------------------------------
+
+extern "C" int smat_device_count(int *n)
+{
+    if (!n) return set_error(SMAT_ERR_INVALID, "n must not be NULL");
+    SMAT_HIP(hipGetDeviceCount(n));
+    return SMAT_OK;
+}
+extern "C" int smat_set_device(int dev) { SMAT_HIP(hipSetDevice(dev)); return SMAT_OK; }
+extern "C" int smat_device_name(int dev, char *buf, size_t len)
+{
+    if (!buf || !len) return set_error(SMAT_ERR_INVALID, "buf must not be NULL");
+    hipDeviceProp_t prop;
+    SMAT_HIP(hipGetDeviceProperties(&prop, dev));
+    snprintf(buf, len, "%s (%s)", prop.name, prop.gcnArchName);
+    return SMAT_OK;
+}
+extern "C" int smat_device_attr(int dev, int64_t *cus, int64_t *lds_bytes, int64_t *mem_bytes,
+                                 int64_t *clock_khz)
+{
+    hipDeviceProp_t prop;
+    SMAT_HIP(hipGetDeviceProperties(&prop, dev));
+    if (cus) *cus = prop.multiProcessorCount;
+    if (lds_bytes) *lds_bytes = (int64_t)prop.maxSharedMemoryPerMultiProcessor;
+    if (mem_bytes) *mem_bytes = (int64_t)prop.totalGlobalMem;
+    if (clock_khz) *clock_khz = prop.clockRate;
+    return SMAT_OK;
+}
+extern "C" int smat_malloc(void **dptr, size_t bytes)
+{
+    if (!dptr) return set_error(SMAT_ERR_INVALID, "dptr must not be NULL");
+    SMAT_HIP(hipMalloc(dptr, bytes ? bytes : 1));
+    return SMAT_OK;
+}
+extern "C" int smat_free(void *dptr) { if (dptr) SMAT_HIP(hipFree(dptr)); return SMAT_OK; }
+extern "C" int smat_memcpy_h2d(void *d, const void *s, size_t n) { if (n) SMAT_HIP(hipMemcpy(d, s, n, hipMemcpyHostToDevice)); return SMAT_OK; }
+extern "C" int smat_memcpy_d2h(void *d, const void *s, size_t n) { if (n) SMAT_HIP(hipMemcpy(d, s, n, hipMemcpyDeviceToHost)); return SMAT_OK; }
+extern "C" int smat_memcpy_d2d(void *d, const void *s, size_t n) { if (n) SMAT_HIP(hipMemcpy(d, s, n, hipMemcpyDeviceToDevice)); return SMAT_OK; }
+extern "C" int smat_memset(void *d, int byte, size_t n) { if (n) SMAT_HIP(hipMemset(d, byte, n)); return SMAT_OK; }
+extern "C" int smat_device_synchronize(void) { SMAT_HIP(hipDeviceSynchronize()); return SMAT_OK; }
+extern "C" int smat_stream_create(void **s)
+{
+    if (!s) return set_error(SMAT_ERR_INVALID, "stream must not be NULL");
+    hipStream_t st;
+    SMAT_HIP(hipStreamCreate(&st)); // default priority
+    *s = st;
+    return SMAT_OK;
+}
+extern "C" int smat_stream_destroy(void *s) { if (s) SMAT_HIP(hipStreamDestroy((hipStream_t)s)); return SMAT_OK; }
+extern "C" int smat_stream_synchronize(void *s) { SMAT_HIP(hipStreamSynchronize((hipStream_t)s)); return SMAT_OK; }
+extern "C" int smat_event_create(void **ev)
+{
+    if (!ev) return set_error(SMAT_ERR_INVALID, "event must not be NULL");
+    hipEvent_t e;
+    SMAT_HIP(hipEventCreate(&e));
+    *ev = e;
+    return SMAT_OK;
+}
+extern "C" int smat_event_destroy(void *ev) { if (ev) SMAT_HIP(hipEventDestroy((hipEvent_t)ev)); return SMAT_OK; }
+extern "C" int smat_event_record(void *ev, void *s) { SMAT_HIP(hipEventRecord((hipEvent_t)ev, (hipStream_t)s)); return SMAT_OK; }
+extern "C" int smat_event_synchronize(void *ev) { SMAT_HIP(hipEventSynchronize((hipEvent_t)ev)); return SMAT_OK; }
+extern "C" int smat_event_elapsed_ms(void *a, void *b, float *ms)
+{
+    if (!ms) return set_error(SMAT_ERR_INVALID, "ms must not be NULL");
+    SMAT_HIP(hipEventElapsedTime(ms, (hipEvent_t)a, (hipEvent_t)b));
+    return SMAT_OK;
+}

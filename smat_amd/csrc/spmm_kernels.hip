@@ -1,0 +1,258 @@
+// Block-sparse SpMM kernels for gfx950 (MI355X): C = A_bcsr(16x16, fp16) * B(fp16),
+// fp32 accumulation on v_mfma_f32_16x16x32_f16.
+//
+// Replaces the reference's live kernel mmaCBTKernelSparse and its launcher
+// (src/cuda_hgemm/src/mma/mmaCBT.cu:13-88).  Same operands and semantics
+// (absolute col_idx, column-major B, row-major C overwritten), different
+// machine mapping:
+//
+//  * The product is formed transposed, C^T = B^T * A^T, so that a lane ends up
+//    owning runs of consecutive C columns of one C row (wide stores) and both
+//    MFMA operands are 16-byte, k-contiguous loads: B^T rows are the columns of
+//    the column-major B, A^T columns are the rows of a row-major 16x16 block.
+//  * One MFMA consumes two nonzero blocks of the same block row (K = 32 = 2x16):
+//    lanes 0-31 feed block p, lanes 32-63 feed block p+1; a pair of blocks is one
+//    contiguous, fully coalesced 1 KiB load.
+//  * Work is a list of (block row, block range) items; block rows longer than
+//    the chunk size are split and their fp32 partial tiles are summed in a fixed
+//    order by a second kernel, so results do not depend on scheduling.
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+#include "spmm_kernels.h"
+
+namespace smat {
+
+typedef _Float16 f16x8 __attribute__((ext_vector_type(8)));
+typedef _Float16 f16x4 __attribute__((ext_vector_type(4)));
+typedef float f32x4 __attribute__((ext_vector_type(4)));
+
+__device__ __forceinline__ f16x8 load_f16x8(const uint16_t *p)
+{
+    return *reinterpret_cast<const f16x8 *>(p);
+}
+
+__device__ __forceinline__ f16x8 zero_f16x8()
+{
+    f16x8 z = {0, 0, 0, 0, 0, 0, 0, 0};
+    return z;
+}
+
+// Column of C owned by MFMA output row i (0..15) of n-tile t inside a wave's
+// panel.  Tiles are taken in groups of TG = min(TN, 4); inside a group the
+// assignment interleaves tiles so that the 4*TG values a lane holds for one C
+// row are consecutive columns.
+template <int TN>
+__device__ __forceinline__ int ncol_of(int t, int i)
+{
+    constexpr int TG = TN < 4 ? TN : 4;
+    return 16 * TG * (t / TG) + 4 * TG * (i >> 2) + 4 * (t % TG) + (i & 3);
+}
+
+// One wavefront per work item x N panel.  blockDim = 256 (4 wavefronts).
+//   items == nullptr : item w is the whole block row w (no work list)
+//   items != nullptr : items[w] = {block row, first block, end block, dst}
+//                      dst < 0  -> write the finished tile to C
+//                      dst >= 0 -> write the fp32 partial tile to workspace slot dst
+// Item index runs fastest inside a panel, so the four wavefronts of a workgroup
+// and neighbouring workgroups share one B panel (K x 16*TN) in L2.  Workgroup
+// ids are dealt round-robin to the 8 XCDs by the dispatcher; the remap below
+// gives each XCD a contiguous eighth of the (panel-major) item space so that an
+// XCD's private L2 holds few distinct B panels.
+template <int TN, bool C_F32>
+__global__ __launch_bounds__(256) void spmm_rowwise_kernel(
+    const uint16_t *__restrict__ vals, const int32_t *__restrict__ row_ptr,
+    const int32_t *__restrict__ col_idx, const uint16_t *__restrict__ B, void *__restrict__ Cout,
+    float *__restrict__ workspace, const WorkItem *__restrict__ items, int n_items, int N, long K,
+    int n_panels)
+{
+    constexpr int TG = TN < 4 ? TN : 4;
+    constexpr int PANEL = 16 * TN;
+    const int lane = threadIdx.x & 63;
+    // wavefront-uniform values are forced into scalar registers
+    const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+
+    const long total = (long)n_items * n_panels;
+    const int chunk = gridDim.x >> 3; // gridDim.x is a multiple of 8
+    const long wg = (long)(blockIdx.x & 7) * chunk + (blockIdx.x >> 3);
+    const long w = wg * 4 + wave;
+    if (w >= total) return;
+    const int panel = (int)(w / n_items);
+    const int it = (int)(w - (long)panel * n_items);
+
+    int br, p0, p1, dst;
+    if (items) {
+        WorkItem wi = items[it];
+        br = wi.block_row; p0 = wi.begin; p1 = wi.end; dst = wi.dst;
+    } else {
+        br = it; p0 = row_ptr[it]; p1 = row_ptr[it + 1]; dst = -1;
+    }
+    br = __builtin_amdgcn_readfirstlane(br);
+    p0 = __builtin_amdgcn_readfirstlane(p0);
+    p1 = __builtin_amdgcn_readfirstlane(p1);
+    dst = __builtin_amdgcn_readfirstlane(dst);
+
+    const int i16 = lane & 15; // A row m / B^T row (n within tile)
+    const int g = lane >> 4;   // k group 0..3
+    const int sel = g >> 1;    // which block of the pair
+    const int kh = g & 1;      // which half (8 k) of the block
+    const int n0 = panel * PANEL;
+
+    f32x4 acc[TN];
+    long boff[TN];
+    bool nok[TN];
+#pragma unroll
+    for (int t = 0; t < TN; t++) {
+        acc[t] = (f32x4){0.f, 0.f, 0.f, 0.f};
+        int n = n0 + ncol_of<TN>(t, i16);
+        nok[t] = n < N;
+        boff[t] = (long)(nok[t] ? n : 0) * K + kh * 8;
+    }
+    const uint16_t *abase = vals + i16 * 16 + kh * 8;
+
+    for (int pb = p0; pb < p1; pb += 64) {
+        const int cnt = (p1 - pb) < 64 ? (p1 - pb) : 64;
+        // one coalesced load of up to 64 column indices, then lane broadcasts
+        const int myc = (lane < cnt) ? col_idx[pb + lane] : 0;
+        for (int j = 0; j < cnt; j += 2) {
+            const int c0 = __builtin_amdgcn_readlane(myc, j);
+            const int c1 = __builtin_amdgcn_readlane(myc, (j + 1) & 63);
+            const bool valid = (sel == 0) || (j + 1 < cnt);
+            const int bc = sel ? c1 : c0;
+            const long pp = (long)pb + j + sel;
+            f16x8 a = valid ? load_f16x8(abase + pp * 256) : zero_f16x8();
+            f16x8 b[TN];
+#pragma unroll
+            for (int t = 0; t < TN; t++)
+                b[t] = (valid && nok[t]) ? load_f16x8(B + boff[t] + bc) : zero_f16x8();
+#pragma unroll
+            for (int t = 0; t < TN; t++)
+                acc[t] = __builtin_amdgcn_mfma_f32_16x16x32_f16(b[t], a, acc[t], 0, 0, 0);
+        }
+    }
+
+    // Epilogue.  acc[t][r] = C[br*16 + i16][n0 + ncol_of(t, 4*g + r)].
+    const long m = (long)br * 16 + i16;
+#pragma unroll
+    for (int u = 0; u < TN / TG; u++) {
+        const int nbase = n0 + 16 * TG * u + 4 * TG * g; // first of 4*TG consecutive columns
+        if (dst >= 0) {
+            // fp32 partial tile: slot-major, then the same row-major M x N addressing
+            float *wrow = workspace + ((long)dst * 16 + i16) * (long)N;
+#pragma unroll
+            for (int tt = 0; tt < TG; tt++) {
+                int n = nbase + 4 * tt;
+                if (n < N) *reinterpret_cast<f32x4 *>(wrow + n) = acc[u * TG + tt];
+            }
+        } else if (C_F32) {
+            float *crow = reinterpret_cast<float *>(Cout) + m * (long)N;
+#pragma unroll
+            for (int tt = 0; tt < TG; tt++) {
+                int n = nbase + 4 * tt;
+                if (n < N) *reinterpret_cast<f32x4 *>(crow + n) = acc[u * TG + tt];
+            }
+        } else {
+            uint16_t *crow = reinterpret_cast<uint16_t *>(Cout) + m * (long)N;
+            if constexpr (TG == 1) {
+                f32x4 v = acc[u];
+                f16x4 h = {(_Float16)v[0], (_Float16)v[1], (_Float16)v[2], (_Float16)v[3]};
+                if (nbase < N) *reinterpret_cast<f16x4 *>(crow + nbase) = h;
+            } else {
+#pragma unroll
+                for (int tt = 0; tt < TG; tt += 2) {
+                    f32x4 v0 = acc[u * TG + tt], v1 = acc[u * TG + tt + 1];
+                    f16x8 h = {(_Float16)v0[0], (_Float16)v0[1], (_Float16)v0[2], (_Float16)v0[3],
+                               (_Float16)v1[0], (_Float16)v1[1], (_Float16)v1[2], (_Float16)v1[3]};
+                    int n = nbase + 4 * tt;
+                    if (n < N) *reinterpret_cast<f16x8 *>(crow + n) = h;
+                }
+            }
+        }
+    }
+}
+
+// Sums the fp32 partial tiles of every split block row in slot order and writes
+// the finished rows to C.  One thread per 4 consecutive columns of one row.
+template <bool C_F32>
+__global__ __launch_bounds__(256) void spmm_reduce_kernel(const float *__restrict__ workspace,
+                                                         const SplitRow *__restrict__ rows,
+                                                         int n_rows, void *__restrict__ Cout, int N)
+{
+    const int quads = N >> 2; // N % 8 == 0
+    const long tid = (long)blockIdx.x * blockDim.x + threadIdx.x;
+    const long per_row = (long)16 * quads;
+    if (tid >= per_row * n_rows) return;
+    const int r = (int)(tid / per_row);
+    const long rem = tid - (long)r * per_row;
+    const int i = (int)(rem / quads);
+    const int q = (int)(rem - (long)i * quads);
+    const SplitRow sr = rows[r];
+    f32x4 s = {0.f, 0.f, 0.f, 0.f};
+    for (int slot = sr.slot_begin; slot < sr.slot_end; slot++)
+        s += *reinterpret_cast<const f32x4 *>(workspace + ((long)slot * 16 + i) * (long)N + 4 * q);
+    const long m = (long)sr.block_row * 16 + i;
+    if (C_F32) {
+        *reinterpret_cast<f32x4 *>(reinterpret_cast<float *>(Cout) + m * (long)N + 4 * q) = s;
+    } else {
+        f16x4 h = {(_Float16)s[0], (_Float16)s[1], (_Float16)s[2], (_Float16)s[3]};
+        *reinterpret_cast<f16x4 *>(reinterpret_cast<uint16_t *>(Cout) + m * (long)N + 4 * q) = h;
+    }
+}
+
+template <int TN>
+static hipError_t launch_rowwise_tn(const SpmmArgs &a, hipStream_t st)
+{
+    const int panel = 16 * TN;
+    const int n_panels = (int)((a.N + panel - 1) / panel);
+    const long total = (long)a.n_items * n_panels;
+    long wgs = (total + 3) / 4;
+    wgs = (wgs + 7) / 8 * 8;
+    if (wgs == 0) return hipSuccess;
+    if (wgs > 0x7fffffffL) return hipErrorInvalidValue;
+    dim3 grid((unsigned)wgs), block(256);
+    if (a.c_f32)
+        hipLaunchKernelGGL((spmm_rowwise_kernel<TN, true>), grid, block, 0, st, a.vals, a.row_ptr,
+                           a.col_idx, a.B, a.C, a.workspace, a.items, a.n_items, (int)a.N,
+                           (long)a.K, n_panels);
+    else
+        hipLaunchKernelGGL((spmm_rowwise_kernel<TN, false>), grid, block, 0, st, a.vals, a.row_ptr,
+                           a.col_idx, a.B, a.C, a.workspace, a.items, a.n_items, (int)a.N,
+                           (long)a.K, n_panels);
+    return hipGetLastError();
+}
+
+int rowwise_panel_tiles(size_t N, int requested)
+{
+    if (requested == 1 || requested == 2 || requested == 4 || requested == 8) return requested;
+    if (N >= 512) return 8;
+    if (N >= 64) return 4;
+    if (N >= 32) return 2;
+    return 1;
+}
+
+hipError_t launch_rowwise(const SpmmArgs &a, hipStream_t st)
+{
+    hipError_t e;
+    switch (rowwise_panel_tiles(a.N, a.panel_tiles)) {
+    case 8: e = launch_rowwise_tn<8>(a, st); break;
+    case 4: e = launch_rowwise_tn<4>(a, st); break;
+    case 2: e = launch_rowwise_tn<2>(a, st); break;
+    default: e = launch_rowwise_tn<1>(a, st); break;
+    }
+    if (e != hipSuccess) return e;
+    if (a.n_split_rows > 0) {
+        const long threads = (long)a.n_split_rows * 16 * (long)(a.N / 4);
+        const long blocks = (threads + 255) / 256;
+        if (blocks > 0x7fffffffL) return hipErrorInvalidValue;
+        if (a.c_f32)
+            hipLaunchKernelGGL((spmm_reduce_kernel<true>), dim3((unsigned)blocks), dim3(256), 0, st,
+                               a.workspace, a.split_rows, a.n_split_rows, a.C, (int)a.N);
+        else
+            hipLaunchKernelGGL((spmm_reduce_kernel<false>), dim3((unsigned)blocks), dim3(256), 0, st,
+                               a.workspace, a.split_rows, a.n_split_rows, a.C, (int)a.N);
+        e = hipGetLastError();
+    }
+    return e;
+}
+
+} // namespace smat

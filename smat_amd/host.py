@@ -1,0 +1,164 @@
+"""Host-side mirror of the reference's matrix-load -> reorder/block -> SpMM flow.
+
+Thin wrappers over the C ABI: numpy arrays for host data, torch CUDA tensors
+(only as device memory) for the SpMM operands.
+"""
+import ctypes as C
+from dataclasses import dataclass
+
+import numpy as np
+
+from ._lib import SpmmOpts, check, lib
+
+BS = 16
+KERNEL_AUTO, KERNEL_ROWWISE, KERNEL_SWEEP = 0, 1, 2
+C_F16, C_F32 = 0, 1
+
+
+def _take(ptr, n, dtype):
+    """Copy n elements out of a library-owned buffer, then free it."""
+    if n:
+        arr = np.ctypeslib.as_array(C.cast(ptr, C.POINTER(np.ctypeslib.as_ctypes_type(dtype))), shape=(n,)).copy()
+    else:
+        arr = np.zeros(0, dtype=dtype)
+    lib.smat_host_free(ptr)
+    return arr
+
+
+def _p(a):
+    return a.ctypes.data_as(C.c_void_p) if a is not None else None
+
+
+def mtx_read(path):
+    """Matrix Market -> CSR (loader semantics of mmio_allinone). Returns dict."""
+    M, K, nnz, sym, ref = C.c_size_t(), C.c_size_t(), C.c_size_t(), C.c_int(), C.c_int()
+    rp, ci, v = C.c_void_p(), C.c_void_p(), C.c_void_p()
+    check(lib.smat_mtx_read(str(path).encode(), C.byref(M), C.byref(K), C.byref(nnz), C.byref(sym),
+                            C.byref(rp), C.byref(ci), C.byref(v), C.byref(ref)))
+    return {
+        "M": M.value, "K": K.value, "nnz": nnz.value, "symmetric": bool(sym.value),
+        "row_ptr": _take(rp, M.value + 1, np.int32),
+        "col_idx": _take(ci, nnz.value, np.int32),
+        "val": _take(v, nnz.value, np.uint16),
+    }
+
+
+@dataclass
+class Bcsr:
+    M: int
+    K: int
+    row_ptr: np.ndarray  # int32 [M/16+1]
+    col_idx: np.ndarray  # int32 [nnzb], absolute first column of each block
+    val: np.ndarray      # uint16 (fp16 bits) [nnzb*256]
+    counts: tuple        # (nonzero, "dense", "sparse") blocks
+    block_info: np.ndarray = None
+    rel_map: np.ndarray = None
+
+    @property
+    def nnzb(self):
+        return int(self.col_idx.shape[0])
+
+
+def csr_to_bcsr(M, K, row_ptr, col_idx, val, want_maps=False):
+    row_ptr = np.ascontiguousarray(row_ptr, dtype=np.int32)
+    col_idx = np.ascontiguousarray(col_idx, dtype=np.int32)
+    val = np.ascontiguousarray(val, dtype=np.uint16)
+    counts = (C.c_int64 * 3)()
+    brp, bci, bv = C.c_void_p(), C.c_void_p(), C.c_void_p()
+    info, rel = C.c_void_p(), C.c_void_p()
+    check(lib.smat_csr_to_bcsr(M, K, _p(row_ptr), _p(col_idx), _p(val), counts, C.byref(brp), C.byref(bci),
+                               C.byref(bv), C.byref(info) if want_maps else None,
+                               C.byref(rel) if want_maps else None))
+    nnzb = counts[0]
+    out = Bcsr(M, K, _take(brp, M // BS + 1, np.int32), _take(bci, nnzb, np.int32),
+               _take(bv, nnzb * 256, np.uint16), tuple(counts))
+    if want_maps:
+        cells = (M // BS) * (K // BS)
+        out.block_info = _take(info, cells, np.int32)
+        out.rel_map = _take(rel, cells, np.int32)
+    return out
+
+
+def reorder_rows(rows, cols, row_ptr, col_idx, col_block=16, row_block=16, tau=0.5):
+    """One pass of the row clustering. Returns (grouping, perm, stats)."""
+    row_ptr = np.ascontiguousarray(row_ptr, dtype=np.int64)
+    col_idx = np.ascontiguousarray(col_idx, dtype=np.int64)
+    grouping = np.empty(rows, dtype=np.int64)
+    perm = np.empty(rows, dtype=np.int64)
+    stats = np.zeros(4, dtype=np.int64)
+    check(lib.smat_reorder_rows(rows, cols, _p(row_ptr), _p(col_idx), col_block, row_block, tau,
+                                _p(grouping), _p(perm), _p(stats)))
+    return grouping, perm, stats
+
+
+def reorder_csr(M, K, row_ptr, col_idx, col_block=16, row_block=16, tau=0.5, do_cols=True):
+    row_ptr = np.ascontiguousarray(row_ptr, dtype=np.int32)
+    col_idx = np.ascontiguousarray(col_idx, dtype=np.int32)
+    pr = np.empty(M, dtype=np.int64)
+    pc = np.empty(K, dtype=np.int64)
+    sr = np.zeros(4, dtype=np.int64)
+    sc = np.zeros(4, dtype=np.int64)
+    check(lib.smat_reorder_csr(M, K, _p(row_ptr), _p(col_idx), col_block, row_block, tau, int(do_cols),
+                               _p(pr), _p(pc), _p(sr), _p(sc)))
+    return pr, pc, sr, sc
+
+
+def permute_csr(M, K, row_ptr, col_idx, val, perm_rows=None, perm_cols=None):
+    row_ptr = np.ascontiguousarray(row_ptr, dtype=np.int32)
+    col_idx = np.ascontiguousarray(col_idx, dtype=np.int32)
+    val = np.ascontiguousarray(val, dtype=np.uint16)
+    pr = None if perm_rows is None else np.ascontiguousarray(perm_rows, dtype=np.int64)
+    pc = None if perm_cols is None else np.ascontiguousarray(perm_cols, dtype=np.int64)
+    orp, oci, ov = C.c_void_p(), C.c_void_p(), C.c_void_p()
+    check(lib.smat_permute_csr(M, K, _p(row_ptr), _p(col_idx), _p(val), _p(pr), _p(pc),
+                               C.byref(orp), C.byref(oci), C.byref(ov)))
+    nnz = int(row_ptr[M])
+    return _take(orp, M + 1, np.int32), _take(oci, nnz, np.int32), _take(ov, nnz, np.uint16)
+
+
+class Plan:
+    """Per-matrix work list (built once, outside any timed loop)."""
+
+    def __init__(self, row_ptr_host, M, K, nnzb, n_hint, col_idx_host=None, kernel=KERNEL_AUTO):
+        self._h = C.c_void_p()
+        rp = np.ascontiguousarray(row_ptr_host, dtype=np.int32)
+        ci = None if col_idx_host is None else np.ascontiguousarray(col_idx_host, dtype=np.int32)
+        opts = SpmmOpts(0, 0, kernel, 0, None)
+        check(lib.smat_plan_create(C.byref(self._h), _p(rp), _p(ci), M, K, nnzb, n_hint, C.byref(opts)))
+
+    @property
+    def handle(self):
+        return self._h
+
+    def info(self):
+        out = (C.c_int64 * 8)()
+        check(lib.smat_plan_info(self._h, out))
+        keys = ("kernel", "items", "split_rows", "chunk", "workspace_bytes", "panel", "_6", "_7")
+        return dict(zip(keys, out))
+
+    def close(self):
+        if self._h:
+            lib.smat_plan_destroy(self._h)
+            self._h = C.c_void_p()
+
+    def __del__(self):
+        try:
+            self.close()
+        except Exception:
+            pass
+
+
+def spmm(vals, row_ptr, col_idx, B, C_out, M, N, K, nnzb, plan=None, c_f32=False, kernel=KERNEL_AUTO,
+         stream=None, drop_in=False):
+    """Launch the SpMM on device tensors (anything with .data_ptr()).
+
+    drop_in=True calls the positional drop-in entry point (smat_spmm_bcsr_f16) with
+    NULL block_info / rel_map; otherwise the options entry point."""
+    ptr = lambda t: C.c_void_p(t.data_ptr()) if t is not None else None  # noqa: E731
+    if drop_in:
+        check(lib.smat_spmm_bcsr_f16(ptr(vals), ptr(row_ptr), ptr(col_idx), ptr(B), ptr(C_out), M, N, K, nnzb,
+                                     None, None))
+        return
+    opts = SpmmOpts(0, C_F32 if c_f32 else C_F16, kernel, 0, C.c_void_p(stream) if stream else None)
+    check(lib.smat_spmm_bcsr_f16_ex(ptr(vals), ptr(row_ptr), ptr(col_idx), ptr(B), ptr(C_out), M, N, K, nnzb,
+                                    C.byref(opts), plan.handle if plan is not None else None))
