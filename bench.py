@@ -1,0 +1,190 @@
+#!/usr/bin/env python3
+"""Headline benchmark: block-sparse SpMM on one MI355X.
+
+A "step" is one SpMM launch C = A_bcsr x B over inputs already resident in HBM.
+Default workload = the block-pruned configuration the metric is quoted on:
+A 8192 x 8192 fp16, 16x16 block mask with 10% of the blocks kept (dense inside,
+N(0, 0.02)), B 8192 x 4096 fp16 N(0,1), fp16 C.  The work list (plan) is built
+once, outside the timed region, like the reference builds its BCSR once.
+
+Prints ONE JSON line: effective GFLOP/s = 2 * nnzb * 256 * N / t, the roofline
+fraction of the SpMM kernel (timed with HIP events on the launch stream), and a
+CPU baseline (the oracle's blocked loop nest on the host cores, bounded sample).
+"""
+import argparse
+import ctypes as C
+import json
+import os
+import sys
+import time
+
+import numpy as np
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+sys.path.insert(0, ROOT)
+
+PEAK_FP16_TFLOPS = 2500.0  # MI355X dense fp16 MFMA
+PEAK_HBM_GBS = 8000.0      # MI355X HBM3E
+
+
+def build_workload(name):
+    from smat_amd import generators as gen
+    import smat_amd
+    if name == "block_pruned_8192_10pct_N4096":
+        A = gen.block_pruned(8192, 0.10, 0.02)
+        N, bdist, bseed = 4096, "normal", 0xB0000004
+    elif name == "band_4096_bw64_N128":
+        d = gen.band(4096, 64)
+        b = smat_amd.csr_to_bcsr(d["M"], d["K"], d["row_ptr"], d["col_idx"], d["val"])
+        A = {"M": b.M, "K": b.K, "b_row_ptr": b.row_ptr, "b_col_idx": b.col_idx, "b_val": b.val, "nnzb": b.nnzb}
+        N, bdist, bseed = 128, "uniform", 0xB0000001
+    elif name == "stencil27_64_N64":
+        d = gen.stencil27(64)
+        b = smat_amd.csr_to_bcsr(d["M"], d["K"], d["row_ptr"], d["col_idx"], d["val"])
+        A = {"M": b.M, "K": b.K, "b_row_ptr": b.row_ptr, "b_col_idx": b.col_idx, "b_val": b.val, "nnzb": b.nnzb}
+        N, bdist, bseed = 64, "uniform", 0xB0000005
+    elif name == "er_16384_0.1pct_N256":
+        d = gen.erdos_renyi(16384, 0.001)
+        b = smat_amd.csr_to_bcsr(d["M"], d["K"], d["row_ptr"], d["col_idx"], d["val"])
+        A = {"M": b.M, "K": b.K, "b_row_ptr": b.row_ptr, "b_col_idx": b.col_idx, "b_val": b.val, "nnzb": b.nnzb}
+        N, bdist, bseed = 256, "normal", 0xB0000002
+    else:
+        raise SystemExit(f"unknown workload {name}")
+    B = gen.dense_b(A["K"], N, seed=bseed, dist=bdist)
+    return A, B, N
+
+
+def algorithmic_bytes(A, N, c_bytes=2):
+    """Every operand touched once: blocks (512 B values + 4 B index), row pointer, B, C."""
+    mb = A["M"] // 16
+    return A["nnzb"] * 516 + (mb + 1) * 4 + 2 * A["K"] * N + c_bytes * A["M"] * N
+
+
+def cpu_baseline(A, B, N, target_s=12.0):
+    """Oracle blocked SpMM (fp32 accumulate) on the host cores over a leading slice of block rows."""
+    from tests.oracle_lib import load_oracle
+    oracle = load_oracle()
+    threads = max(1, min(16, os.cpu_count() or 1, oracle.max_threads()))
+    rp = A["b_row_ptr"]
+    mb = A["M"] // 16
+
+    def run(nrows):
+        sub_rp = rp[:nrows + 1].astype(np.int32)
+        nb = int(sub_rp[-1])
+        t0 = time.perf_counter()
+        oracle.spmm_bcsr(16 * nrows, N, A["K"], sub_rp, A["b_col_idx"][:nb], A["b_val"][:nb * 256], B,
+                         threads=threads)
+        return time.perf_counter() - t0, nb
+
+    probe_rows = min(mb, 2 * threads)
+    t_probe, nb_probe = run(probe_rows)
+    # the widening of B to fp32 is a fixed cost of the oracle; the sample is sized on the loop nest
+    rows = int(min(mb, max(probe_rows, probe_rows * target_s / max(t_probe, 1e-3))))
+    t, nb = run(rows)
+    gflops = 2.0 * nb * 256 * N / t / 1e9
+    return {"value": round(gflops, 3), "unit": "GFLOP/s", "cores": threads, "kind": "port",
+            "sample": f"first {rows} of {mb} block rows ({nb} blocks) of the same workload, {t:.2f} s, "
+                      f"OpenMP over block rows, includes widening B to fp32"}
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=200)
+    ap.add_argument("--warmup", type=int, default=20)
+    ap.add_argument("--workload", default="block_pruned_8192_10pct_N4096")
+    ap.add_argument("--kernel", type=int, default=0, help="0 auto, 1 rowwise, 2 sweep")
+    ap.add_argument("--no-plan", action="store_true")
+    ap.add_argument("--no-cpu-baseline", action="store_true")
+    args = ap.parse_args()
+    if args.gpus != 1:
+        raise SystemExit("bench.py measures one MI355X: run with --gpus 1 (this build has no multi-GPU path)")
+
+    import torch
+    import smat_amd
+    from smat_amd._lib import lib, check
+
+    assert torch.cuda.is_available(), "bench.py needs a GPU"
+    dev = torch.device("cuda:0")
+    A, B, N = build_workload(args.workload)
+    M, K, nnzb = A["M"], A["K"], A["nnzb"]
+
+    def dev_i16(a):
+        return torch.from_numpy(np.ascontiguousarray(a).view(np.int16)).to(dev)
+
+    vals, Bd = dev_i16(A["b_val"]), dev_i16(B)
+    rp = torch.from_numpy(A["b_row_ptr"].astype(np.int32)).to(dev)
+    ci = torch.from_numpy(A["b_col_idx"].astype(np.int32)).to(dev)
+    Cd = torch.zeros((M, N), dtype=torch.int16, device=dev)
+    plan = None
+    if not args.no_plan:
+        plan = smat_amd.Plan(A["b_row_ptr"], M, K, nnzb, N, col_idx_host=A["b_col_idx"], kernel=args.kernel)
+
+    def step():
+        smat_amd.spmm(vals, rp, ci, Bd, Cd, M, N, K, nnzb, plan=plan, kernel=args.kernel)
+
+    for _ in range(args.warmup):
+        step()
+    torch.cuda.synchronize()
+
+    # HIP events on the stream the kernels are launched on (the null stream)
+    ev0, ev1 = C.c_void_p(), C.c_void_p()
+    check(lib.smat_event_create(C.byref(ev0)))
+    check(lib.smat_event_create(C.byref(ev1)))
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    check(lib.smat_event_record(ev0, None))
+    for _ in range(args.steps):
+        step()
+    check(lib.smat_event_record(ev1, None))
+    check(lib.smat_event_synchronize(ev1))
+    torch.cuda.synchronize()
+    wall_ms = (time.perf_counter() - t0) * 1e3 / args.steps
+    ms = C.c_float()
+    check(lib.smat_event_elapsed_ms(ev0, ev1, C.byref(ms)))
+    kernel_ms = ms.value / args.steps
+    lib.smat_event_destroy(ev0)
+    lib.smat_event_destroy(ev1)
+
+    flops = 2.0 * nnzb * 256 * N
+    qbytes = algorithmic_bytes(A, N)
+    value = flops / (wall_ms * 1e-3) / 1e9
+    ach_tflops = flops / (kernel_ms * 1e-3) / 1e12
+    ach_gbs = qbytes / (kernel_ms * 1e-3) / 1e9
+    mfma_bound = (flops / (PEAK_FP16_TFLOPS * 1e12)) >= (qbytes / (PEAK_HBM_GBS * 1e9))
+    if mfma_bound:
+        roof = {"bound": "mfma", "achieved": round(ach_tflops, 2), "peak": PEAK_FP16_TFLOPS, "unit": "TFLOP/s",
+                "frac": round(ach_tflops / PEAK_FP16_TFLOPS, 4)}
+    else:
+        roof = {"bound": "hbm", "achieved": round(ach_gbs, 1), "peak": PEAK_HBM_GBS, "unit": "GB/s",
+                "frac": round(ach_gbs / PEAK_HBM_GBS, 4)}
+    roof["traffic"] = None
+    roof["kernel_ms"] = round(kernel_ms, 5)
+    roof["algorithmic_flops"] = flops
+    roof["algorithmic_bytes"] = qbytes
+    roof["hbm_gbs_at_algorithmic_bytes"] = round(ach_gbs, 1)
+
+    out = {
+        "metric": "effective SpMM GFLOP/s + % of fp16 MFMA/HBM roofline, 1x MI355X",
+        "value": round(value, 1),
+        "unit": "GFLOP/s",
+        "n_gpus": 1,
+        "steps": args.steps,
+        "warmup": args.warmup,
+        "ms_per_step": round(wall_ms, 5),
+        "higher_is_better": True,
+        "scaling": "weak",
+        "vs_baseline": None,
+        "dtype": "f16",
+        "data": "synthetic",
+        "config": {"workload": args.workload, "M": M, "K": K, "N": N, "nnzb": nnzb, "block": 16,
+                   "c_dtype": "f16", "plan": None if plan is None else plan.info()},
+        "roofline": roof,
+    }
+    if not args.no_cpu_baseline:
+        out["cpu_baseline"] = cpu_baseline(A, B, N)
+    print(json.dumps(out))
+
+
+if __name__ == "__main__":
+    main()

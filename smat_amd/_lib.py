@@ -74,6 +74,13 @@ def _load():
             f"{path} is missing: build it with `python -c 'import __graft_entry__ as g; g.build()'` "
             "(or `make -C smat_amd/csrc`). There is no CPU fallback."
         )
+    # PyTorch wheels carry their own HIP runtime (same SONAME as the system one).  Two
+    # runtimes in one process cannot both open the GPU, so when torch is installed it
+    # is imported first and this library binds to the runtime torch already loaded.
+    try:
+        import torch  # noqa: F401
+    except ImportError:
+        pass
     handle = C.CDLL(path)
     for name, (res, args) in SIGNATURES.items():
         fn = getattr(handle, name)

@@ -1,0 +1,218 @@
+"""GPU parity tests: the HIP SpMM, called through the C ABI, against the CPU oracle.
+
+Bar: max_j |C[i][j] - ref[i][j]| / ||ref[i][:]||_2 <= 1e-3 for the fp16 output
+(the tolerance the port's acceptance criterion states), and <= 2e-6 for the
+fp32-output variant (only the summation order differs from the oracle)."""
+import numpy as np
+import pytest
+
+from smat_amd import generators as gen
+
+pytestmark = pytest.mark.gpu
+
+TOL_F16 = 1e-3
+TOL_F32 = 2e-6
+
+
+def to_dev(torch, arr, device):
+    a = np.ascontiguousarray(arr)
+    if a.dtype == np.uint16:
+        return torch.from_numpy(a.view(np.int16)).to(device)
+    return torch.from_numpy(a).to(device)
+
+
+def gpu_spmm(smat, cuda, A, B_bits, N, plan=False, c_f32=False, drop_in=False, poison=True):
+    """A: dict with M, K, b_row_ptr, b_col_idx, b_val. Returns C as numpy (uint16 bits or float32)."""
+    import torch
+    M, K, nnzb = A["M"], A["K"], int(A["b_col_idx"].shape[0])
+    vals = to_dev(torch, A["b_val"] if nnzb else np.zeros(8, np.uint16), cuda)
+    rp = to_dev(torch, A["b_row_ptr"].astype(np.int32), cuda)
+    ci = to_dev(torch, A["b_col_idx"].astype(np.int32) if nnzb else np.zeros(1, np.int32), cuda)
+    B = to_dev(torch, B_bits, cuda)
+    if c_f32:
+        C = torch.full((M, N), float("nan") if poison else 0.0, dtype=torch.float32, device=cuda)
+    else:
+        C = torch.full((M, N), 0x7E00 if poison else 0, dtype=torch.int16, device=cuda)  # fp16 NaN pattern
+    p = None
+    if plan:
+        p = smat.Plan(A["b_row_ptr"], M, K, nnzb, N, col_idx_host=A["b_col_idx"])
+    torch.cuda.synchronize()
+    smat.spmm(vals, rp, ci, B, C, M, N, K, nnzb, plan=p, c_f32=c_f32, drop_in=drop_in)
+    torch.cuda.synchronize()
+    out = C.cpu().numpy()
+    if p is not None:
+        p.close()
+    return out if c_f32 else out.view(np.uint16)
+
+
+def rel_err_f32(c, ref):
+    nrm = np.sqrt((ref.astype(np.float64) ** 2).sum(axis=1))
+    nrm[nrm == 0] = 1.0
+    d = np.abs(c.astype(np.float64) - ref.astype(np.float64)).max(axis=1)
+    return float((d / nrm).max())
+
+
+def oracle_ref(oracle, A, B_bits, N):
+    return oracle.spmm_bcsr(A["M"], N, A["K"], A["b_row_ptr"], A["b_col_idx"], A["b_val"], B_bits, threads=8)
+
+
+def test_single_identity_block_gathers_b_rows(smat, cuda, oracle):
+    # A = one 16x16 identity block at block column 2 of a 16 x 64 matrix: C = B[32:48, :]
+    eye = np.eye(16, dtype=np.float16).view(np.uint16).ravel()
+    A = {"M": 16, "K": 64, "b_row_ptr": np.array([0, 1], np.int32), "b_col_idx": np.array([32], np.int32),
+         "b_val": eye}
+    for N in (8, 16, 24, 64, 136):
+        B = gen.dense_b(64, N, seed=7, dist="uniform")
+        C = gpu_spmm(smat, cuda, A, B, N)
+        expect = B.reshape(N, 64).T[32:48, :]  # column-major B: element (k, n) at [n*K + k]
+        assert np.array_equal(C, expect), f"N={N}"
+
+
+def test_asymmetric_block_pins_operand_orientation(smat, cuda, oracle):
+    # one block with a single nonzero at (row 3, col 11): C[3, :] = 2 * B[16*1 + 11, :], all else 0
+    blk = np.zeros((16, 16), dtype=np.float16)
+    blk[3, 11] = 2.0
+    A = {"M": 32, "K": 48, "b_row_ptr": np.array([0, 0, 1], np.int32), "b_col_idx": np.array([16], np.int32),
+         "b_val": blk.view(np.uint16).ravel()}
+    N = 40
+    B = gen.dense_b(48, N, seed=9, dist="uniform")
+    C = gpu_spmm(smat, cuda, A, B, N).view(np.float16).astype(np.float32)
+    Bm = B.view(np.float16).reshape(N, 48).T.astype(np.float32)
+    expect = np.zeros((32, N), dtype=np.float32)
+    expect[16 + 3, :] = 2.0 * Bm[16 + 11, :]
+    assert np.array_equal(C, expect)
+
+
+@pytest.mark.parametrize("N", [8, 16, 24, 32, 40, 64, 72, 128, 136, 256, 520, 1032])
+def test_random_bcsr_all_panel_widths(smat, cuda, oracle, N):
+    A = gen.random_bcsr(9, 13, 0.35, seed=100 + N)
+    B = gen.dense_b(A["K"], N, seed=200 + N, dist="normal")
+    ref = oracle_ref(oracle, A, B, N)
+    C = gpu_spmm(smat, cuda, A, B, N)
+    err = oracle.compare(C, ref)[0]
+    assert err <= TOL_F16, (N, err)
+    C32 = gpu_spmm(smat, cuda, A, B, N, c_f32=True)
+    assert rel_err_f32(C32, ref) <= TOL_F32
+    # the fp16 output is exactly the rounded fp32 output
+    assert np.array_equal(C32.astype(np.float16).view(np.uint16), C)
+
+
+def test_drop_in_entry_matches_options_entry(smat, cuda, oracle):
+    A = gen.random_bcsr(20, 20, 0.2, seed=5)
+    N = 96
+    B = gen.dense_b(A["K"], N, seed=6)
+    c1 = gpu_spmm(smat, cuda, A, B, N, drop_in=True)
+    c2 = gpu_spmm(smat, cuda, A, B, N, drop_in=False)
+    assert np.array_equal(c1, c2)
+    assert oracle.compare(c1, oracle_ref(oracle, A, B, N))[0] <= TOL_F16
+
+
+def test_empty_matrix_and_empty_rows_write_zeros(smat, cuda, oracle):
+    N = 72
+    B = gen.dense_b(64, N, seed=1)
+    empty = {"M": 48, "K": 64, "b_row_ptr": np.zeros(4, np.int32), "b_col_idx": np.zeros(0, np.int32),
+             "b_val": np.zeros(0, np.uint16)}
+    assert not gpu_spmm(smat, cuda, empty, B, N).any()
+    assert not gpu_spmm(smat, cuda, empty, B, N, plan=True).any()
+    A = gen.random_bcsr(6, 4, 0.0, seed=2, row_lengths=[0, 3, 0, 0, 1, 0])
+    ref = oracle_ref(oracle, A, B, N)
+    for plan in (False, True):
+        C = gpu_spmm(smat, cuda, A, B, N, plan=plan)
+        assert oracle.compare(C, ref)[0] <= TOL_F16
+        assert not C.reshape(A["M"], N)[0:16].any() and not C.reshape(A["M"], N)[32:64].any()
+
+
+@pytest.mark.parametrize("lengths", [
+    [1, 2, 3, 4, 5, 63, 64, 65, 127, 128, 129, 0],   # odd/even tails, 64-block index refills
+    [700, 1, 1, 1, 0, 2, 1, 1, 3, 1, 1, 1, 1, 1, 1, 1],  # one very long row: split by the plan
+    [300, 290, 2, 2, 2, 2, 2, 2, 2, 2, 2, 2, 2, 2, 2, 2, 2, 2, 2, 2],  # two long rows
+])
+def test_skewed_rows_with_and_without_plan(smat, cuda, oracle, lengths):
+    kb = max(max(lengths), 8)
+    A = gen.random_bcsr(len(lengths), kb, 0.0, seed=len(lengths), row_lengths=lengths)
+    N = 88
+    B = gen.dense_b(A["K"], N, seed=33)
+    ref = oracle_ref(oracle, A, B, N)
+    c0 = gpu_spmm(smat, cuda, A, B, N, plan=False)
+    c1 = gpu_spmm(smat, cuda, A, B, N, plan=True)
+    assert oracle.compare(c0, ref)[0] <= TOL_F16
+    assert oracle.compare(c1, ref)[0] <= TOL_F16
+    c32 = gpu_spmm(smat, cuda, A, B, N, plan=True, c_f32=True)
+    assert rel_err_f32(c32, ref) <= TOL_F32
+
+
+def test_plan_splits_long_rows(smat, cuda):
+    lengths = [700] + [1] * 15
+    A = gen.random_bcsr(16, 700, 0.0, seed=3, row_lengths=lengths)
+    p = smat.Plan(A["b_row_ptr"], A["M"], A["K"], A["nnzb"], 64)
+    info = p.info()
+    p.close()
+    assert info["split_rows"] == 1 and info["items"] > 16 and info["workspace_bytes"] > 0
+
+
+def test_b_ones_gives_row_sums(smat, cuda, oracle):
+    # the reference fills B with 1.0 (common/matrix.h:38): every column of C is the row sum of A
+    A = gen.random_bcsr(12, 12, 0.4, seed=77)
+    N = 48
+    B = np.full(A["K"] * N, 0x3C00, dtype=np.uint16)
+    C = gpu_spmm(smat, cuda, A, B, N, c_f32=True)
+    rp, ci, v = gen.bcsr_to_csr(A["M"], A["b_row_ptr"], A["b_col_idx"], A["b_val"])
+    sums = np.zeros(A["M"], dtype=np.float64)
+    np.add.at(sums, np.repeat(np.arange(A["M"]), np.diff(rp)), v.view(np.float16).astype(np.float64))
+    assert np.allclose(C, sums[:, None], rtol=0, atol=1e-4)
+    assert (C == C[:, :1]).all()
+
+
+def test_config1_band_full_size(smat, cuda, oracle):
+    d = gen.band(4096, 64)
+    A = smat.csr_to_bcsr(d["M"], d["K"], d["row_ptr"], d["col_idx"], d["val"])
+    assert A.nnzb == 2284
+    Ad = {"M": A.M, "K": A.K, "b_row_ptr": A.row_ptr, "b_col_idx": A.col_idx, "b_val": A.val}
+    N = 128
+    B = gen.dense_b(A.K, N, seed=0xB0000001, dist="uniform")
+    ref = oracle.spmm_csr(d["M"], N, d["K"], d["row_ptr"], d["col_idx"], d["val"], B)  # from CSR: independent of blocking
+    for plan in (False, True):
+        C = gpu_spmm(smat, cuda, Ad, B, N, plan=plan)
+        assert oracle.compare(C, ref)[0] <= TOL_F16
+
+
+def test_config5_stencil_reduced_and_reordered(smat, cuda, oracle):
+    d = gen.stencil27(16)  # 4096 rows
+    N = 64
+    B = gen.dense_b(d["K"], N, seed=0xB0000005, dist="uniform")
+    ref = oracle.spmm_csr(d["M"], N, d["K"], d["row_ptr"], d["col_idx"], d["val"], B)
+    A = smat.csr_to_bcsr(d["M"], d["K"], d["row_ptr"], d["col_idx"], d["val"])
+    Ad = {"M": A.M, "K": A.K, "b_row_ptr": A.row_ptr, "b_col_idx": A.col_idx, "b_val": A.val}
+    C = gpu_spmm(smat, cuda, Ad, B, N, plan=True)
+    assert oracle.compare(C, ref)[0] <= TOL_F16
+    # reordered: P_r A P_c^T applied to P_c B gives P_r C
+    pr, pc, _, _ = smat.reorder_csr(d["M"], d["K"], d["row_ptr"], d["col_idx"])
+    rp2, ci2, v2 = smat.permute_csr(d["M"], d["K"], d["row_ptr"], d["col_idx"], d["val"], pr, pc)
+    A2 = smat.csr_to_bcsr(d["M"], d["K"], rp2, ci2, v2)
+    Bm = B.reshape(N, d["K"])
+    B2 = np.ascontiguousarray(Bm[:, pc]).ravel()
+    A2d = {"M": A2.M, "K": A2.K, "b_row_ptr": A2.row_ptr, "b_col_idx": A2.col_idx, "b_val": A2.val}
+    C2 = gpu_spmm(smat, cuda, A2d, B2, N, plan=True)
+    assert oracle.compare(C2, ref[pr])[0] <= TOL_F16
+
+
+def test_config4_block_pruned_full_size_sampled_rows(smat, cuda, oracle):
+    A = gen.block_pruned(8192, 0.10, 0.02)
+    assert A["nnzb"] == 26214
+    N = 4096
+    B = gen.dense_b(8192, N, seed=0xB0000004, dist="normal")
+    C = gpu_spmm(smat, cuda, A, B, N, plan=True).reshape(8192, N)
+    # oracle on a sample of block rows (the full product is ~3e10 MACs on the CPU)
+    rows = [0, 1, 17, 255, 256, 300, 511]
+    rp = A["b_row_ptr"]
+    sel = np.concatenate([np.arange(rp[r], rp[r + 1]) for r in rows])
+    sub = {"M": 16 * len(rows), "K": 8192,
+           "b_row_ptr": np.concatenate([[0], np.cumsum([rp[r + 1] - rp[r] for r in rows])]).astype(np.int32),
+           "b_col_idx": A["b_col_idx"][sel],
+           "b_val": A["b_val"].reshape(-1, 256)[sel].ravel()}
+    ref = oracle_ref(oracle, sub, B, N)
+    got = np.concatenate([C[16 * r:16 * r + 16] for r in rows])
+    assert oracle.compare(got, ref)[0] <= TOL_F16
+    # size-independent property: an independent launch without a plan gives the identical bits
+    C2 = gpu_spmm(smat, cuda, A, B, N, plan=False).reshape(8192, N)
+    assert np.array_equal(C, C2)
