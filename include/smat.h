@@ -88,8 +88,8 @@ typedef struct smat_plan smat_plan;
 int smat_plan_create(smat_plan **plan, const int32_t *row_ptr_host, const int32_t *col_idx_host,
                      size_t M, size_t K, size_t nnzb, size_t n_hint, const smat_spmm_opts *opts);
 int smat_plan_destroy(smat_plan *plan);
-/* Fills info[0..7]: kernel id, work items, split block rows, chunk size,
- * workspace bytes, panel width, 0, 0. */
+/* Fills info[0..7]: kernel id, row-wise work items, split block rows, chunk size,
+ * workspace bytes, panel width, sweep MFMA ops, sweep (row group, K chunk) records. */
 int smat_plan_info(const smat_plan *plan, int64_t *info);
 
 /* Same operands as smat_spmm_bcsr_f16; C is uint16_t* or float* per opts->c_dtype.

@@ -34,6 +34,10 @@ struct smat_plan {
     SplitRow *d_split = nullptr;
     float *d_workspace = nullptr;
     size_t workspace_bytes = 0;
+    // sweep kernel work list (present when kernel == SMAT_KERNEL_SWEEP)
+    int n_rg = 0, n_records = 0, n_ops = 0;
+    int32_t *d_rg_chunk_ptr = nullptr, *d_chunk_ids = nullptr, *d_op_ptr = nullptr;
+    SweepOp *d_ops = nullptr;
 };
 
 extern "C" const char *smat_version(void) { return "smat-amd 0.1 gfx950"; }
@@ -89,7 +93,22 @@ extern "C" int smat_spmm_bcsr_f16_ex(const uint16_t *vals, const int32_t *row_pt
         a.workspace = plan->d_workspace;
         a.panel_tiles = plan->panel_tiles;
     }
-    hipError_t e = launch_rowwise(a, static_cast<hipStream_t>(o.stream));
+    int kernel = o.kernel;
+    if (kernel == SMAT_KERNEL_AUTO) kernel = plan ? plan->kernel : SMAT_KERNEL_ROWWISE;
+    if (kernel != SMAT_KERNEL_ROWWISE && kernel != SMAT_KERNEL_SWEEP)
+        return set_error(SMAT_ERR_INVALID, "unknown kernel id %d", kernel);
+    hipError_t e;
+    if (kernel == SMAT_KERNEL_SWEEP) {
+        if (!plan || !plan->d_ops)
+            return set_error(SMAT_ERR_INVALID, "SMAT_KERNEL_SWEEP needs a plan built for it (with col_idx_host)");
+        SweepArgs w{};
+        w.vals = vals; w.B = B; w.C = C; w.M = M; w.N = N; w.K = K; w.c_f32 = a.c_f32;
+        w.rg_chunk_ptr = plan->d_rg_chunk_ptr; w.chunk_ids = plan->d_chunk_ids;
+        w.op_ptr = plan->d_op_ptr; w.ops = plan->d_ops; w.n_rg = plan->n_rg;
+        e = launch_sweep(w, static_cast<hipStream_t>(o.stream));
+    } else {
+        e = launch_rowwise(a, static_cast<hipStream_t>(o.stream));
+    }
     if (e != hipSuccess)
         return set_error(SMAT_ERR_HIP, "SpMM launch failed: %s", hipGetErrorString(e));
     return SMAT_OK;
@@ -111,7 +130,6 @@ extern "C" int smat_plan_create(smat_plan **out, const int32_t *row_ptr_host,
                                  const int32_t *col_idx_host, size_t M, size_t K, size_t nnzb,
                                  size_t n_hint, const smat_spmm_opts *opts)
 {
-    (void)col_idx_host;
     if (!out || !row_ptr_host) return set_error(SMAT_ERR_INVALID, "plan and row_ptr_host must not be NULL");
     if (M == 0 || M % 16 || K % 16) return set_error(SMAT_ERR_INVALID, "M and K must be positive multiples of 16");
     if (n_hint == 0 || n_hint % 8) return set_error(SMAT_ERR_INVALID, "n_hint must be a positive multiple of 8");
@@ -121,8 +139,15 @@ extern "C" int smat_plan_create(smat_plan **out, const int32_t *row_ptr_host,
     for (size_t i = 0; i < mb; i++)
         if (row_ptr_host[i + 1] < row_ptr_host[i])
             return set_error(SMAT_ERR_INVALID, "row_ptr_host must be non-decreasing");
-    if (opts && opts->kernel == SMAT_KERNEL_SWEEP)
-        return set_error(SMAT_ERR_UNSUPPORTED, "SMAT_KERNEL_SWEEP is not implemented");
+    const int want = opts ? opts->kernel : SMAT_KERNEL_AUTO;
+    if (want == SMAT_KERNEL_SWEEP && !col_idx_host)
+        return set_error(SMAT_ERR_INVALID, "SMAT_KERNEL_SWEEP needs col_idx_host");
+    const size_t kb = K / 16;
+    if (col_idx_host)
+        for (size_t p = 0; p < nnzb; p++)
+            if (col_idx_host[p] < 0 || col_idx_host[p] % 16 || (size_t)col_idx_host[p] >= K)
+                return set_error(SMAT_ERR_INVALID, "col_idx_host[%zu] = %d is not a block column of K = %zu",
+                                 p, col_idx_host[p], K);
 
     smat_plan *p = new (std::nothrow) smat_plan();
     if (!p) return set_error(SMAT_ERR_NOMEM, "out of host memory");
@@ -173,6 +198,72 @@ extern "C" int smat_plan_create(smat_plan **out, const int32_t *row_ptr_host,
         p->workspace_bytes = (size_t)slot * 16 * n_hint * sizeof(float);
         if (e == hipSuccess) e = hipMalloc(&p->d_workspace, p->workspace_bytes);
     }
+    // The sweep kernel pays one pass over the B panel per group of 32 block rows,
+    // whatever the sparsity: worth it only when a few percent of the blocks exist
+    // and N is wide.
+    bool sweep = want == SMAT_KERNEL_SWEEP;
+    if (want == SMAT_KERNEL_AUTO && col_idx_host && n_hint >= 128 && mb >= (size_t)SWEEP_G &&
+        (double)nnzb >= 0.02 * (double)mb * (double)kb)
+        sweep = true;
+    if (e == hipSuccess && sweep) {
+        const size_t n_rg = (mb + SWEEP_G - 1) / SWEEP_G;
+        std::vector<int32_t> rg_ptr(n_rg + 1, 0), chunk_ids, op_ptr(1, 0);
+        std::vector<SweepOp> ops;
+        struct Ent { int32_t chunk, wave, r, slab, p; };
+        std::vector<Ent> ents;
+        for (size_t rg = 0; rg < n_rg; rg++) {
+            ents.clear();
+            const size_t r_end = std::min(mb, (rg + 1) * SWEEP_G);
+            for (size_t br = rg * SWEEP_G; br < r_end; br++) {
+                const int local = (int)(br - rg * SWEEP_G);
+                for (int32_t q = row_ptr_host[br]; q < row_ptr_host[br + 1]; q++) {
+                    const int32_t bc = col_idx_host[q] / 16;
+                    ents.push_back(Ent{bc / SWEEP_S, local / SWEEP_RW, local % SWEEP_RW, bc % SWEEP_S, q});
+                }
+            }
+            std::sort(ents.begin(), ents.end(), [](const Ent &x, const Ent &y) {
+                if (x.chunk != y.chunk) return x.chunk < y.chunk;
+                if (x.wave != y.wave) return x.wave < y.wave;
+                if (x.r != y.r) return x.r < y.r;
+                return x.slab < y.slab;
+            });
+            size_t i = 0;
+            while (i < ents.size()) {
+                const int32_t chunk = ents[i].chunk;
+                chunk_ids.push_back(chunk);
+                for (int w = 0; w < SWEEP_WAVES; w++)
+                    for (int r = 0; r < SWEEP_RW; r++) {
+                        while (i < ents.size() && ents[i].chunk == chunk && ents[i].wave == w && ents[i].r == r) {
+                            const bool pair = i + 1 < ents.size() && ents[i + 1].chunk == chunk &&
+                                              ents[i + 1].wave == w && ents[i + 1].r == r;
+                            SweepOp op;
+                            op.p1 = ents[i].p;
+                            op.p2 = pair ? ents[i + 1].p : -1;
+                            // a single block feeds the upper MFMA half with zeros of A and the same slab
+                            op.meta = (ents[i].slab << 8) | ((pair ? ents[i + 1].slab : ents[i].slab) << 16);
+                            op.pad = 0;
+                            ops.push_back(op);
+                            i += pair ? 2 : 1;
+                        }
+                        op_ptr.push_back((int32_t)ops.size());
+                    }
+            }
+            rg_ptr[rg + 1] = (int32_t)chunk_ids.size();
+        }
+        p->kernel = SMAT_KERNEL_SWEEP;
+        p->n_rg = (int)n_rg;
+        p->n_records = (int)chunk_ids.size();
+        p->n_ops = (int)ops.size();
+        auto upload = [&](void **dst, const void *src, size_t bytes) {
+            if (e != hipSuccess) return;
+            e = hipMalloc(dst, std::max<size_t>(bytes, 16));
+            if (e == hipSuccess && bytes) e = hipMemcpy(*dst, src, bytes, hipMemcpyHostToDevice);
+        };
+        upload((void **)&p->d_rg_chunk_ptr, rg_ptr.data(), rg_ptr.size() * sizeof(int32_t));
+        upload((void **)&p->d_chunk_ids, chunk_ids.data(), chunk_ids.size() * sizeof(int32_t));
+        upload((void **)&p->d_op_ptr, op_ptr.data(), op_ptr.size() * sizeof(int32_t));
+        upload((void **)&p->d_ops, ops.data(), ops.size() * sizeof(SweepOp));
+    }
     if (e != hipSuccess) {
         smat_plan_destroy(p);
         return set_error(SMAT_ERR_HIP, "plan allocation failed: %s", hipGetErrorString(e));
@@ -187,6 +278,10 @@ extern "C" int smat_plan_destroy(smat_plan *p)
     if (p->d_items) (void)hipFree(p->d_items);
     if (p->d_split) (void)hipFree(p->d_split);
     if (p->d_workspace) (void)hipFree(p->d_workspace);
+    if (p->d_rg_chunk_ptr) (void)hipFree(p->d_rg_chunk_ptr);
+    if (p->d_chunk_ids) (void)hipFree(p->d_chunk_ids);
+    if (p->d_op_ptr) (void)hipFree(p->d_op_ptr);
+    if (p->d_ops) (void)hipFree(p->d_ops);
     delete p;
     return SMAT_OK;
 }
@@ -195,7 +290,9 @@ extern "C" int smat_plan_info(const smat_plan *p, int64_t *info)
 {
     if (!p || !info) return set_error(SMAT_ERR_INVALID, "plan and info must not be NULL");
     info[0] = p->kernel; info[1] = p->n_items; info[2] = p->n_split_rows; info[3] = p->chunk;
-    info[4] = (int64_t)p->workspace_bytes; info[5] = 16 * p->panel_tiles; info[6] = 0; info[7] = 0;
+    info[4] = (int64_t)p->workspace_bytes;
+    info[5] = p->kernel == SMAT_KERNEL_SWEEP ? 16 * SWEEP_TN : 16 * p->panel_tiles;
+    info[6] = p->n_ops; info[7] = p->n_records;
     return SMAT_OK;
 }
 

@@ -39,7 +39,39 @@ struct SpmmArgs {
     float *workspace; // device, n_slots * 16 * N floats
 };
 
+// One MFMA worth of work in the sweep kernel: two blocks of the same block row
+// whose block columns lie in the same K chunk (p2 < 0: a single block).
+// meta = slab of p1 << 8 | slab of p2 << 16, slab = block column
+// relative to the first block column of the chunk.
+struct SweepOp {
+    int32_t p1;
+    int32_t p2;
+    int32_t meta;
+    int32_t pad;
+};
+
+// Geometry of the sweep kernel (fixed at compile time).
+constexpr int SWEEP_TN = 8;     // n-tiles of 16 per workgroup panel -> 128 columns
+constexpr int SWEEP_RW = 4;     // block rows per wavefront
+constexpr int SWEEP_WAVES = 8;  // wavefronts per workgroup
+constexpr int SWEEP_G = SWEEP_RW * SWEEP_WAVES; // 32 block rows per workgroup
+constexpr int SWEEP_S = 16;     // block columns (slabs) per K chunk
+
+struct SweepArgs {
+    const uint16_t *vals;
+    const uint16_t *B;
+    void *C;
+    size_t M, N, K;
+    bool c_f32;
+    const int32_t *rg_chunk_ptr; // device, n_rg + 1: range of (row group, chunk) records
+    const int32_t *chunk_ids;    // device, chunk index of each record
+    const int32_t *op_ptr;       // device, records * SWEEP_WAVES * SWEEP_RW + 1
+    const SweepOp *ops;          // device
+    int n_rg;
+};
+
 int rowwise_panel_tiles(size_t N, int requested);
+hipError_t launch_sweep(const SweepArgs &a, hipStream_t st);
 hipError_t launch_rowwise(const SpmmArgs &a, hipStream_t st);
 
 } // namespace smat

@@ -1,0 +1,233 @@
+// "Sweep" SpMM kernel for block matrices that are dense enough (a few percent of
+// the 16x16 blocks present) and wide N: one workgroup owns a group of 32 block
+// rows x 128 columns of C and sweeps over K in chunks of 16 block columns.
+//
+//  * The B panel of a chunk (256 k x 128 n, 64 KiB) is staged once per workgroup
+//    in LDS and shared by all block rows of the group; global reads of it are
+//    256-byte contiguous runs of the column-major B (B[n*K + k]), i.e. fully
+//    used cache lines, instead of the 32-byte gathers a per-block read costs.
+//  * LDS holds a chunk as [8-slab group][n][16 slots of 16 B]; a slot is 8
+//    consecutive k of one n.  The slot index is XOR-ed with a 4-bit function of
+//    n chosen so that the 16 lanes of one ds_read_b128 phase (which read 16
+//    different n, same logical slot) hit 16 different 16-byte bank groups, and
+//    the 16 lanes that fill one n write 256 contiguous bytes: no bank conflicts
+//    on either side.
+//  * Each wavefront owns 4 block rows (128 fp32 accumulator registers) and runs
+//    a host-built list of MFMA ops, grouped by block row so that the accumulator
+//    registers of an op are known at compile time: pairs of blocks of one block row inside the
+//    chunk feed one v_mfma_f32_16x16x32_f16 (K = 32 = 2 blocks).  A operands are
+//    512-byte coalesced global reads straight into MFMA layout.
+//  * Two LDS stages: chunk c+1 is copied global -> LDS asynchronously
+//    (global_load_lds_dwordx4, no staging registers) while the MFMA work of
+//    chunk c runs; one barrier per chunk.
+//
+// Same operand semantics as the reference launcher
+// (src/cuda_hgemm/src/mma/mmaCBT.cu:83-88).
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+#include "spmm_kernels.h"
+
+namespace smat {
+
+typedef _Float16 f16x8 __attribute__((ext_vector_type(8)));
+typedef float f32x4 __attribute__((ext_vector_type(4)));
+
+namespace {
+
+constexpr int TN = SWEEP_TN, RW = SWEEP_RW, W = SWEEP_WAVES, S = SWEEP_S;
+constexpr int NT = 16 * TN;                 // 128 columns per panel
+constexpr int THREADS = 64 * W;             // 512
+constexpr int OCTS = S / 8;                 // 8-slab groups per chunk
+constexpr int ROW_BYTES = 256;              // 8 slabs x 16 k x 2 B per n
+constexpr int STAGE_BYTES = OCTS * NT * ROW_BYTES; // 65536
+constexpr int FILL_ITERS = STAGE_BYTES / 16 / THREADS; // 16-byte slots per thread per chunk: 8
+
+// LDS slot swizzle: physical slot = logical slot ^ ((n & 3) | ((n >> 2) & 12)), n = column in the panel.
+
+// Issues the asynchronous global -> LDS copies of one chunk of the B panel into
+// `stage`.  One wave instruction moves 64 x 16 B = 1 KiB: four n-rows of 256 B.
+// LDS destination = wave-uniform base + lane * 16 (hardware addressing of
+// global_load_lds_dwordx4); the global source is per lane, so the XOR swizzle is
+// applied on the source side.  Columns beyond N are skipped (their LDS rows only
+// feed C columns that are never stored) and k is clamped into the matrix (slabs
+// past K are referenced by no op).
+__device__ __forceinline__ void fill_issue(unsigned char *stage, const uint16_t *__restrict__ B,
+                                           int chunk, int n0, int N, long K, int wave, int lane)
+{
+    // Instruction `it` of wavefront `wave` covers rows (it*W + wave)*4 .. +3 of the
+    // stage, i.e. slab group o = it/4 and n = (it%4)*32 + wave*4 + lane/16.
+    static_assert(W == 8 && NT == 128 && FILL_ITERS == 8, "fill mapping assumes 8 waves x 128 columns");
+    const int q = lane >> 4, ps = lane & 15;
+    // swizzle_of_n(n) = q | bit4(n) << 2 | bit5(n) << 3 with bit4(n) = wave/4, bit5(n) = it & 1
+    const int ls0 = ps ^ (q | (((wave >> 2) & 1) << 2));
+    const long kmax = K - 8;
+#pragma unroll
+    for (int it = 0; it < FILL_ITERS; it++) {
+        const int nrow = n0 + (it & 3) * 32 + wave * 4; // first of 4 columns, wave-uniform
+        if (nrow >= N) continue;                          // N % 8 == 0: all four or none
+        const int ls = ls0 ^ ((it & 1) << 3);
+        long k = (long)chunk * (S * 16) + (it >> 2) * 128 + ls * 8;
+        k = k < kmax ? k : kmax; // slabs past K are never referenced; keep the read in bounds
+        const uint16_t *src = B + (long)(nrow + q) * K + k;
+        __builtin_amdgcn_global_load_lds(
+            (const __attribute__((address_space(1))) void *)src,
+            (__attribute__((address_space(3))) void *)(stage + (size_t)(it * W + wave) * 1024), 16, 0, 0);
+    }
+}
+
+} // namespace
+
+template <bool C_F32>
+__global__ __launch_bounds__(THREADS) void spmm_sweep_kernel(
+    const uint16_t *__restrict__ vals, const uint16_t *__restrict__ B, void *__restrict__ Cout,
+    const int32_t *__restrict__ rg_chunk_ptr, const int32_t *__restrict__ chunk_ids,
+    const int32_t *__restrict__ op_ptr, const SweepOp *__restrict__ ops, int Mb, int N, long K,
+    int n_rg, int n_panels)
+{
+    extern __shared__ __align__(16) unsigned char lds[];
+
+    const int tid = threadIdx.x;
+    const int lane = tid & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+
+    // panel-major work order, row group fastest; each XCD gets a contiguous eighth
+    const int total = n_rg * n_panels;
+    const int per_xcd = gridDim.x >> 3;
+    const int wg = (blockIdx.x & 7) * per_xcd + (blockIdx.x >> 3);
+    if (wg >= total) return;
+    const int panel = wg / n_rg;
+    const int rg = wg - panel * n_rg;
+    const int n0 = panel * NT;
+
+    const int i16 = lane & 15, g = lane >> 4, sel = g >> 1, kh = g & 1;
+    // column (within the panel) of MFMA row i16 in tile 0; tile t adds 64*(t/4) + 4*(t%4)
+    const int n_lane = 16 * (i16 >> 2) + (i16 & 3);
+    const int rd_base = n_lane * ROW_BYTES; // swizzle_of_n(n_lane + tile offset) == i16 for every tile
+
+    f32x4 acc[RW][TN];
+#pragma unroll
+    for (int r = 0; r < RW; r++)
+#pragma unroll
+        for (int t = 0; t < TN; t++) acc[r][t] = (f32x4){0.f, 0.f, 0.f, 0.f};
+
+    const int c_begin = rg_chunk_ptr[rg], c_end = rg_chunk_ptr[rg + 1];
+    const uint16_t *abase = vals + i16 * 16 + kh * 8;
+    const f16x8 zero8 = {0, 0, 0, 0, 0, 0, 0, 0};
+
+    int stage = 0;
+    if (c_begin < c_end) fill_issue(lds, B, chunk_ids[c_begin], n0, N, K, wave, lane);
+    __builtin_amdgcn_s_waitcnt(0x0f70); // vmcnt(0): the copies of this wavefront have landed
+    __syncthreads();
+
+    for (int ci = c_begin; ci < c_end; ci++) {
+        // ops of this wavefront in this chunk, grouped by local block row r:
+        // [op_ptr[base + r], op_ptr[base + r + 1])
+        const int base = (ci * W + wave) * RW;
+        const int o_first = op_ptr[base], o_last = op_ptr[base + RW];
+        SweepOp op = {0, -1, 0, 0};
+        f16x8 a = zero8;
+        if (o_first < o_last) { // A operand of the first op: issued ahead of the B copies
+            op = ops[o_first];
+            const int p = sel ? op.p2 : op.p1;
+            a = p >= 0 ? *reinterpret_cast<const f16x8 *>(abase + (long)p * 256) : zero8;
+        }
+        const bool more = ci + 1 < c_end;
+        if (more) fill_issue(lds + (stage ^ 1) * STAGE_BYTES, B, chunk_ids[ci + 1], n0, N, K, wave, lane);
+
+        const unsigned char *cur = lds + stage * STAGE_BYTES + rd_base;
+#pragma unroll
+        for (int r = 0; r < RW; r++) {
+            const int o_end = op_ptr[base + r + 1];
+            for (int o = op_ptr[base + r]; o < o_end; o++) {
+                SweepOp opn = {0, -1, 0, 0};
+                f16x8 an = zero8;
+                if (o + 1 < o_last) { // next op of this wavefront (possibly of the next row)
+                    opn = ops[o + 1];
+                    const int p = sel ? opn.p2 : opn.p1;
+                    an = p >= 0 ? *reinterpret_cast<const f16x8 *>(abase + (long)p * 256) : zero8;
+                }
+                const int s = sel ? ((op.meta >> 16) & 0xff) : ((op.meta >> 8) & 0xff);
+                const int swz = (s >> 3) * (NT * ROW_BYTES) + (((((s & 7) << 1) | kh) ^ i16) << 4);
+                const unsigned char *bp = cur + swz;
+#pragma unroll
+                for (int u = 0; u < TN / 4; u++) {
+                    f16x8 b[4];
+#pragma unroll
+                    for (int tt = 0; tt < 4; tt++)
+                        b[tt] = *reinterpret_cast<const f16x8 *>(bp + (64 * u + 4 * tt) * ROW_BYTES);
+#pragma unroll
+                    for (int tt = 0; tt < 4; tt++)
+                        acc[r][u * 4 + tt] = __builtin_amdgcn_mfma_f32_16x16x32_f16(
+                            b[tt], a, acc[r][u * 4 + tt], 0, 0, 0);
+                }
+                op = opn;
+                a = an;
+            }
+        }
+        __builtin_amdgcn_s_waitcnt(0x0f70); // vmcnt(0): this wavefront's copies have landed
+        __syncthreads();
+        stage ^= 1;
+    }
+
+    // Epilogue: acc[r][t][e] = C[(rg*G + wave*RW + r)*16 + i16][n0 + 64*(t/4) + 16*g + 4*(t%4) + e]
+#pragma unroll
+    for (int r = 0; r < RW; r++) {
+        const int br = rg * SWEEP_G + wave * RW + r;
+        if (br >= Mb) continue;
+        const long m = (long)br * 16 + i16;
+#pragma unroll
+        for (int u = 0; u < TN / 4; u++) {
+            const int nbase = n0 + 64 * u + 16 * g;
+            if (C_F32) {
+                float *crow = reinterpret_cast<float *>(Cout) + m * (long)N;
+#pragma unroll
+                for (int tt = 0; tt < 4; tt++)
+                    if (nbase + 4 * tt < N)
+                        *reinterpret_cast<f32x4 *>(crow + nbase + 4 * tt) = acc[r][u * 4 + tt];
+            } else {
+                uint16_t *crow = reinterpret_cast<uint16_t *>(Cout) + m * (long)N;
+#pragma unroll
+                for (int tt = 0; tt < 4; tt += 2) {
+                    const f32x4 v0 = acc[r][u * 4 + tt], v1 = acc[r][u * 4 + tt + 1];
+                    f16x8 h = {(_Float16)v0[0], (_Float16)v0[1], (_Float16)v0[2], (_Float16)v0[3],
+                               (_Float16)v1[0], (_Float16)v1[1], (_Float16)v1[2], (_Float16)v1[3]};
+                    if (nbase + 4 * tt < N) *reinterpret_cast<f16x8 *>(crow + nbase + 4 * tt) = h;
+                }
+            }
+        }
+    }
+}
+
+hipError_t launch_sweep(const SweepArgs &a, hipStream_t st)
+{
+    static bool attr_set[2] = {false, false};
+    const int lds_bytes = 2 * STAGE_BYTES;
+    const int which = a.c_f32 ? 1 : 0;
+    if (!attr_set[which]) {
+        hipError_t e = a.c_f32
+            ? hipFuncSetAttribute(reinterpret_cast<const void *>(&spmm_sweep_kernel<true>),
+                                  hipFuncAttributeMaxDynamicSharedMemorySize, lds_bytes)
+            : hipFuncSetAttribute(reinterpret_cast<const void *>(&spmm_sweep_kernel<false>),
+                                  hipFuncAttributeMaxDynamicSharedMemorySize, lds_bytes);
+        if (e != hipSuccess) return e;
+        attr_set[which] = true;
+    }
+    const int n_panels = (int)((a.N + NT - 1) / NT);
+    long wgs = (long)a.n_rg * n_panels;
+    wgs = (wgs + 7) / 8 * 8;
+    if (wgs == 0) return hipSuccess;
+    if (wgs > 0x7fffffffL) return hipErrorInvalidValue;
+    dim3 grid((unsigned)wgs), block(THREADS);
+    if (a.c_f32)
+        hipLaunchKernelGGL((spmm_sweep_kernel<true>), grid, block, lds_bytes, st, a.vals, a.B, a.C,
+                           a.rg_chunk_ptr, a.chunk_ids, a.op_ptr, a.ops, (int)(a.M / 16), (int)a.N,
+                           (long)a.K, a.n_rg, n_panels);
+    else
+        hipLaunchKernelGGL((spmm_sweep_kernel<false>), grid, block, lds_bytes, st, a.vals, a.B, a.C,
+                           a.rg_chunk_ptr, a.chunk_ids, a.op_ptr, a.ops, (int)(a.M / 16), (int)a.N,
+                           (long)a.K, a.n_rg, n_panels);
+    return hipGetLastError();
+}
+
+} // namespace smat

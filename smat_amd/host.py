@@ -133,7 +133,7 @@ class Plan:
     def info(self):
         out = (C.c_int64 * 8)()
         check(lib.smat_plan_info(self._h, out))
-        keys = ("kernel", "items", "split_rows", "chunk", "workspace_bytes", "panel", "_6", "_7")
+        keys = ("kernel", "items", "split_rows", "chunk", "workspace_bytes", "panel", "sweep_ops", "sweep_records")
         return dict(zip(keys, out))
 
     def close(self):

@@ -21,7 +21,7 @@ def to_dev(torch, arr, device):
     return torch.from_numpy(a).to(device)
 
 
-def gpu_spmm(smat, cuda, A, B_bits, N, plan=False, c_f32=False, drop_in=False, poison=True):
+def gpu_spmm(smat, cuda, A, B_bits, N, plan=False, c_f32=False, drop_in=False, poison=True, kernel=0):
     """A: dict with M, K, b_row_ptr, b_col_idx, b_val. Returns C as numpy (uint16 bits or float32)."""
     import torch
     M, K, nnzb = A["M"], A["K"], int(A["b_col_idx"].shape[0])
@@ -35,9 +35,9 @@ def gpu_spmm(smat, cuda, A, B_bits, N, plan=False, c_f32=False, drop_in=False, p
         C = torch.full((M, N), 0x7E00 if poison else 0, dtype=torch.int16, device=cuda)  # fp16 NaN pattern
     p = None
     if plan:
-        p = smat.Plan(A["b_row_ptr"], M, K, nnzb, N, col_idx_host=A["b_col_idx"])
+        p = smat.Plan(A["b_row_ptr"], M, K, nnzb, N, col_idx_host=A["b_col_idx"], kernel=kernel)
     torch.cuda.synchronize()
-    smat.spmm(vals, rp, ci, B, C, M, N, K, nnzb, plan=p, c_f32=c_f32, drop_in=drop_in)
+    smat.spmm(vals, rp, ci, B, C, M, N, K, nnzb, plan=p, c_f32=c_f32, drop_in=drop_in, kernel=kernel)
     torch.cuda.synchronize()
     out = C.cpu().numpy()
     if p is not None:
@@ -150,6 +150,44 @@ def test_plan_splits_long_rows(smat, cuda):
     assert info["split_rows"] == 1 and info["items"] > 16 and info["workspace_bytes"] > 0
 
 
+SWEEP = 2
+
+
+@pytest.mark.parametrize("mb,kb,density,N", [
+    (9, 13, 0.35, 128),     # fewer block rows than one row group, one partial K chunk
+    (40, 40, 0.15, 136),    # partial last panel, partial last row group
+    (64, 33, 0.10, 256),    # K = 528: last chunk is 1 slab wide
+    (33, 70, 0.05, 520),    # sparse enough that some (row group, chunk) records are empty
+    (32, 16, 1.00, 128),    # fully dense: every op is a pair
+])
+def test_sweep_kernel_matches_oracle(smat, cuda, oracle, mb, kb, density, N):
+    A = gen.random_bcsr(mb, kb, density, seed=1000 + mb + kb)
+    B = gen.dense_b(A["K"], N, seed=2000 + N, dist="normal")
+    ref = oracle_ref(oracle, A, B, N)
+    C = gpu_spmm(smat, cuda, A, B, N, plan=True, kernel=SWEEP)
+    assert oracle.compare(C, ref)[0] <= TOL_F16
+    C32 = gpu_spmm(smat, cuda, A, B, N, plan=True, kernel=SWEEP, c_f32=True)
+    assert rel_err_f32(C32, ref) <= TOL_F32
+    assert np.array_equal(C32.astype(np.float16).view(np.uint16), C)
+
+
+def test_sweep_kernel_skewed_and_empty_rows(smat, cuda, oracle):
+    lengths = [0, 90, 1, 0, 0, 3, 2, 64, 0, 17] + [0] * 30 + [5, 90]
+    A = gen.random_bcsr(len(lengths), 90, 0.0, seed=4, row_lengths=lengths)
+    N = 264
+    B = gen.dense_b(A["K"], N, seed=8)
+    ref = oracle_ref(oracle, A, B, N)
+    C = gpu_spmm(smat, cuda, A, B, N, plan=True, kernel=SWEEP)
+    assert oracle.compare(C, ref)[0] <= TOL_F16
+    assert not C.reshape(A["M"], N)[0:16].any()
+
+
+def test_sweep_needs_a_plan_with_col_idx(smat, cuda):
+    A = gen.random_bcsr(4, 4, 0.5, seed=1)
+    with pytest.raises(smat.SmatError):
+        smat.Plan(A["b_row_ptr"], A["M"], A["K"], A["nnzb"], 128, col_idx_host=None, kernel=SWEEP)
+
+
 def test_b_ones_gives_row_sums(smat, cuda, oracle):
     # the reference fills B with 1.0 (common/matrix.h:38): every column of C is the row sum of A
     A = gen.random_bcsr(12, 12, 0.4, seed=77)
@@ -201,7 +239,7 @@ def test_config4_block_pruned_full_size_sampled_rows(smat, cuda, oracle):
     assert A["nnzb"] == 26214
     N = 4096
     B = gen.dense_b(8192, N, seed=0xB0000004, dist="normal")
-    C = gpu_spmm(smat, cuda, A, B, N, plan=True).reshape(8192, N)
+    C = gpu_spmm(smat, cuda, A, B, N, plan=True, kernel=1).reshape(8192, N)
     # oracle on a sample of block rows (the full product is ~3e10 MACs on the CPU)
     rows = [0, 1, 17, 255, 256, 300, 511]
     rp = A["b_row_ptr"]
@@ -216,3 +254,10 @@ def test_config4_block_pruned_full_size_sampled_rows(smat, cuda, oracle):
     # size-independent property: an independent launch without a plan gives the identical bits
     C2 = gpu_spmm(smat, cuda, A, B, N, plan=False).reshape(8192, N)
     assert np.array_equal(C, C2)
+    # the sweep kernel (the plan's own choice for this matrix) pairs blocks differently, so its
+    # fp32 sums may round differently: same tolerance against the oracle, and close to the other kernel
+    C3 = gpu_spmm(smat, cuda, A, B, N, plan=True).reshape(8192, N)
+    got3 = np.concatenate([C3[16 * r:16 * r + 16] for r in rows])
+    assert oracle.compare(got3, ref)[0] <= TOL_F16
+    d = np.abs(C3.view(np.float16).astype(np.float32) - C.view(np.float16).astype(np.float32)).max()
+    assert d <= 2e-3 * np.abs(C.view(np.float16).astype(np.float32)).max()
