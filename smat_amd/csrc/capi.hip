@@ -36,7 +36,7 @@ struct smat_plan {
     size_t workspace_bytes = 0;
     // sweep kernel work list (present when kernel == SMAT_KERNEL_SWEEP)
     int n_rg = 0, n_records = 0, n_ops = 0;
-    int32_t *d_rg_chunk_ptr = nullptr, *d_chunk_ids = nullptr, *d_op_ptr = nullptr;
+    int32_t *d_rg_chunk_ptr = nullptr, *d_chunk_ids = nullptr;
     SweepOp *d_ops = nullptr;
 };
 
@@ -104,7 +104,7 @@ extern "C" int smat_spmm_bcsr_f16_ex(const uint16_t *vals, const int32_t *row_pt
         SweepArgs w{};
         w.vals = vals; w.B = B; w.C = C; w.M = M; w.N = N; w.K = K; w.c_f32 = a.c_f32;
         w.rg_chunk_ptr = plan->d_rg_chunk_ptr; w.chunk_ids = plan->d_chunk_ids;
-        w.op_ptr = plan->d_op_ptr; w.ops = plan->d_ops; w.n_rg = plan->n_rg;
+        w.ops = plan->d_ops; w.n_rg = plan->n_rg;
         e = launch_sweep(w, static_cast<hipStream_t>(o.stream));
     } else {
         e = launch_rowwise(a, static_cast<hipStream_t>(o.stream));
@@ -205,12 +205,23 @@ extern "C" int smat_plan_create(smat_plan **out, const int32_t *row_ptr_host,
     if (want == SMAT_KERNEL_AUTO && col_idx_host && n_hint >= 128 && mb >= (size_t)SWEEP_G &&
         (double)nnzb >= 0.02 * (double)mb * (double)kb)
         sweep = true;
+    if (sweep && nnzb >= (size_t)1 << 23) { // the sweep kernel addresses blocks with 32-bit byte offsets
+        if (want == SMAT_KERNEL_SWEEP) {
+            smat_plan_destroy(p);
+            return set_error(SMAT_ERR_UNSUPPORTED, "SMAT_KERNEL_SWEEP supports fewer than 2^23 nonzero blocks");
+        }
+        sweep = false;
+    }
     if (e == hipSuccess && sweep) {
         const size_t n_rg = (mb + SWEEP_G - 1) / SWEEP_G;
-        std::vector<int32_t> rg_ptr(n_rg + 1, 0), chunk_ids, op_ptr(1, 0);
-        std::vector<SweepOp> ops;
+        std::vector<int32_t> rg_ptr(n_rg + 1, 0), chunk_ids;
+        std::vector<SweepOp> ops; // records * SWEEP_WAVES * SWEEP_CAP table slots
+        const SweepOp empty_slot = {-1, -1, 0, 0};
         struct Ent { int32_t chunk, wave, r, slab, p; };
         std::vector<Ent> ents;
+        constexpr int CAPR = SWEEP_CAP / SWEEP_RW; // table slots per block row
+        std::vector<SweepOp> per_row[SWEEP_WAVES][SWEEP_RW];
+        size_t n_ops = 0;
         for (size_t rg = 0; rg < n_rg; rg++) {
             ents.clear();
             const size_t r_end = std::min(mb, (rg + 1) * SWEEP_G);
@@ -230,30 +241,46 @@ extern "C" int smat_plan_create(smat_plan **out, const int32_t *row_ptr_host,
             size_t i = 0;
             while (i < ents.size()) {
                 const int32_t chunk = ents[i].chunk;
-                chunk_ids.push_back(chunk);
+                size_t most = 0;
                 for (int w = 0; w < SWEEP_WAVES; w++)
                     for (int r = 0; r < SWEEP_RW; r++) {
+                        std::vector<SweepOp> &list = per_row[w][r];
+                        list.clear();
                         while (i < ents.size() && ents[i].chunk == chunk && ents[i].wave == w && ents[i].r == r) {
                             const bool pair = i + 1 < ents.size() && ents[i + 1].chunk == chunk &&
                                               ents[i + 1].wave == w && ents[i + 1].r == r;
                             SweepOp op;
                             op.p1 = ents[i].p;
                             op.p2 = pair ? ents[i + 1].p : -1;
-                            // a single block feeds the upper MFMA half with zeros of A and the same slab
-                            op.meta = (ents[i].slab << 8) | ((pair ? ents[i + 1].slab : ents[i].slab) << 16);
+                            // a single block: the upper MFMA half gets zeros of A and reads the same slab
+                            auto lds_off = [](int32_t slab) { return (slab / 8) * (16 * SWEEP_TN * 256) + (slab % 8) * 32; };
+                            op.meta = lds_off(ents[i].slab) | (lds_off(pair ? ents[i + 1].slab : ents[i].slab) << 16);
                             op.pad = 0;
-                            ops.push_back(op);
+                            list.push_back(op);
                             i += pair ? 2 : 1;
                         }
-                        op_ptr.push_back((int32_t)ops.size());
+                        most = std::max(most, list.size());
+                        n_ops += list.size();
                     }
+                // one record per CAPR ops of the busiest block row; records after the first
+                // reuse the B stage that is already resident
+                const size_t n_rec = (most + CAPR - 1) / CAPR;
+                for (size_t rec = 0; rec < n_rec; rec++) {
+                    chunk_ids.push_back(rec == 0 ? chunk : (chunk | SWEEP_CONT_FLAG));
+                    for (int w = 0; w < SWEEP_WAVES; w++)
+                        for (int r = 0; r < SWEEP_RW; r++)
+                            for (int j = 0; j < CAPR; j++) {
+                                const size_t idx = rec * CAPR + j;
+                                ops.push_back(idx < per_row[w][r].size() ? per_row[w][r][idx] : empty_slot);
+                            }
+                }
             }
             rg_ptr[rg + 1] = (int32_t)chunk_ids.size();
         }
         p->kernel = SMAT_KERNEL_SWEEP;
         p->n_rg = (int)n_rg;
         p->n_records = (int)chunk_ids.size();
-        p->n_ops = (int)ops.size();
+        p->n_ops = (int)n_ops;
         auto upload = [&](void **dst, const void *src, size_t bytes) {
             if (e != hipSuccess) return;
             e = hipMalloc(dst, std::max<size_t>(bytes, 16));
@@ -261,7 +288,6 @@ extern "C" int smat_plan_create(smat_plan **out, const int32_t *row_ptr_host,
         };
         upload((void **)&p->d_rg_chunk_ptr, rg_ptr.data(), rg_ptr.size() * sizeof(int32_t));
         upload((void **)&p->d_chunk_ids, chunk_ids.data(), chunk_ids.size() * sizeof(int32_t));
-        upload((void **)&p->d_op_ptr, op_ptr.data(), op_ptr.size() * sizeof(int32_t));
         upload((void **)&p->d_ops, ops.data(), ops.size() * sizeof(SweepOp));
     }
     if (e != hipSuccess) {
@@ -280,7 +306,6 @@ extern "C" int smat_plan_destroy(smat_plan *p)
     if (p->d_workspace) (void)hipFree(p->d_workspace);
     if (p->d_rg_chunk_ptr) (void)hipFree(p->d_rg_chunk_ptr);
     if (p->d_chunk_ids) (void)hipFree(p->d_chunk_ids);
-    if (p->d_op_ptr) (void)hipFree(p->d_op_ptr);
     if (p->d_ops) (void)hipFree(p->d_ops);
     delete p;
     return SMAT_OK;

@@ -40,9 +40,11 @@ struct SpmmArgs {
 };
 
 // One MFMA worth of work in the sweep kernel: two blocks of the same block row
-// whose block columns lie in the same K chunk (p2 < 0: a single block).
-// meta = slab of p1 << 8 | slab of p2 << 16, slab = block column
-// relative to the first block column of the chunk.
+// whose block columns lie in the same K chunk (p2 < 0: a single block; p1 < 0: an
+// empty table slot).  meta = LDS byte offset of p1's slab | that of p2's slab << 16,
+// offset = (slab / 8) * 128 * 256 + (slab % 8) * 32 with slab = block column
+// relative to the first block column of the chunk (a single repeats p1's slab).
+// Table slot k of a (record, wavefront) serves local block row k / (SWEEP_CAP / SWEEP_RW).
 struct SweepOp {
     int32_t p1;
     int32_t p2;
@@ -56,6 +58,9 @@ constexpr int SWEEP_RW = 4;     // block rows per wavefront
 constexpr int SWEEP_WAVES = 8;  // wavefronts per workgroup
 constexpr int SWEEP_G = SWEEP_RW * SWEEP_WAVES; // 32 block rows per workgroup
 constexpr int SWEEP_S = 16;     // block columns (slabs) per K chunk
+constexpr int SWEEP_CAP = 8;    // op table slots per (record, wavefront): SWEEP_CAP / SWEEP_RW per block row
+
+constexpr int SWEEP_CONT_FLAG = 1 << 30; // chunk_ids bit: record continues the previous record's chunk
 
 struct SweepArgs {
     const uint16_t *vals;
@@ -64,9 +69,9 @@ struct SweepArgs {
     size_t M, N, K;
     bool c_f32;
     const int32_t *rg_chunk_ptr; // device, n_rg + 1: range of (row group, chunk) records
-    const int32_t *chunk_ids;    // device, chunk index of each record
-    const int32_t *op_ptr;       // device, records * SWEEP_WAVES * SWEEP_RW + 1
-    const SweepOp *ops;          // device
+    const int32_t *chunk_ids;    // device, chunk index of each record; SWEEP_CONT_FLAG marks a
+                                 // record that continues the chunk of the record before it
+    const SweepOp *ops;          // device, records * SWEEP_WAVES * SWEEP_CAP table slots
     int n_rg;
 };
 

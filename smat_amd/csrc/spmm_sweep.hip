@@ -13,13 +13,19 @@
 //    the 16 lanes that fill one n write 256 contiguous bytes: no bank conflicts
 //    on either side.
 //  * Each wavefront owns 4 block rows (128 fp32 accumulator registers) and runs
-//    a host-built list of MFMA ops, grouped by block row so that the accumulator
-//    registers of an op are known at compile time: pairs of blocks of one block row inside the
-//    chunk feed one v_mfma_f32_16x16x32_f16 (K = 32 = 2 blocks).  A operands are
-//    512-byte coalesced global reads straight into MFMA layout.
-//  * Two LDS stages: chunk c+1 is copied global -> LDS asynchronously
-//    (global_load_lds_dwordx4, no staging registers) while the MFMA work of
-//    chunk c runs; one barrier per chunk.
+//    a host-built table of MFMA ops with a fixed number of slots per block row
+//    (so the accumulator registers of every slot are known at compile time):
+//    pairs of blocks of one block row inside the chunk feed one
+//    v_mfma_f32_16x16x32_f16 (K = 32 = 2 blocks).  A chunk whose ops do not fit
+//    the table continues in a following record that reuses the resident B stage.  A operands are 512-byte coalesced global reads
+//    straight into MFMA layout.
+//  * Software pipeline over chunks, everything for chunk c+1 is issued before the
+//    MFMA work of chunk c starts and is only waited for after it: the op table of
+//    chunk c+2, the A operands of chunk c+1 (into a second set of registers) and
+//    the B panel of chunk c+1 (global -> LDS asynchronously with
+//    global_load_lds_dwordx4, no staging registers, into the other LDS stage).
+//    The MFMA loop itself touches only registers and LDS.  One barrier per chunk.
+
 //
 // Same operand semantics as the reference launcher
 // (src/cuda_hgemm/src/mma/mmaCBT.cu:83-88).
@@ -70,22 +76,40 @@ __device__ __forceinline__ void fill_issue(unsigned char *stage, const uint16_t 
         long k = (long)chunk * (S * 16) + (it >> 2) * 128 + ls * 8;
         k = k < kmax ? k : kmax; // slabs past K are never referenced; keep the read in bounds
         const uint16_t *src = B + (long)(nrow + q) * K + k;
-        __builtin_amdgcn_global_load_lds(
-            (const __attribute__((address_space(1))) void *)src,
-            (__attribute__((address_space(3))) void *)(stage + (size_t)(it * W + wave) * 1024), 16, 0, 0);
+        // Issued from inline assembly on purpose: the compiler orders every later LDS
+        // read after a global->LDS copy it knows about (it cannot tell the two stages
+        // apart) and would wait for the copy before the MFMA work of the current
+        // chunk.  The copies are waited for explicitly (vmcnt(0)) before the barrier.
+        const uint32_t dst = (uint32_t)(uintptr_t)(__attribute__((address_space(3))) void *)(
+            stage + (size_t)(it * W + wave) * 1024);
+        asm volatile("s_mov_b32 m0, %1\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, off"
+                     :
+                     : "v"(src), "s"(dst)
+                     : "memory", "m0");
     }
 }
 
 } // namespace
 
+typedef int i32x4 __attribute__((ext_vector_type(4)));
+
+// Lane l of the returned vector holds slot l % CAP of the op table of (record,
+// wavefront).  Every lane loads (no branch): a load inside a branch cannot be
+// counted by the compiler's vmcnt bookkeeping and would force full waits later.
+__device__ __forceinline__ i32x4 load_op_table(const SweepOp *__restrict__ ops, int record, int wave, int lane)
+{
+    return *reinterpret_cast<const i32x4 *>(ops + ((long)record * W + wave) * SWEEP_CAP +
+                                            (lane & (SWEEP_CAP - 1)));
+}
+
 template <bool C_F32>
 __global__ __launch_bounds__(THREADS) void spmm_sweep_kernel(
     const uint16_t *__restrict__ vals, const uint16_t *__restrict__ B, void *__restrict__ Cout,
     const int32_t *__restrict__ rg_chunk_ptr, const int32_t *__restrict__ chunk_ids,
-    const int32_t *__restrict__ op_ptr, const SweepOp *__restrict__ ops, int Mb, int N, long K,
-    int n_rg, int n_panels)
+    const SweepOp *__restrict__ ops, int Mb, int N, long K, int n_rg, int n_panels)
 {
     extern __shared__ __align__(16) unsigned char lds[];
+    constexpr int CAP = SWEEP_CAP;
 
     const int tid = threadIdx.x;
     const int lane = tid & 63;
@@ -101,9 +125,11 @@ __global__ __launch_bounds__(THREADS) void spmm_sweep_kernel(
     const int n0 = panel * NT;
 
     const int i16 = lane & 15, g = lane >> 4, sel = g >> 1, kh = g & 1;
-    // column (within the panel) of MFMA row i16 in tile 0; tile t adds 64*(t/4) + 4*(t%4)
+    // column (within the panel) of MFMA row i16 in tile 0; tile t adds 64*(t/4) + 4*(t%4).
+    // The swizzle value of every such column equals i16.
     const int n_lane = 16 * (i16 >> 2) + (i16 & 3);
-    const int rd_base = n_lane * ROW_BYTES; // swizzle_of_n(n_lane + tile offset) == i16 for every tile
+    const int rd_base = n_lane * ROW_BYTES;
+    const uint32_t lane_xor = (uint32_t)((kh ^ i16) << 4); // ((2*slab | kh) ^ i16) << 4 == (slab * 32) ^ lane_xor
 
     f32x4 acc[RW][TN];
 #pragma unroll
@@ -112,64 +138,134 @@ __global__ __launch_bounds__(THREADS) void spmm_sweep_kernel(
         for (int t = 0; t < TN; t++) acc[r][t] = (f32x4){0.f, 0.f, 0.f, 0.f};
 
     const int c_begin = rg_chunk_ptr[rg], c_end = rg_chunk_ptr[rg + 1];
-    const uint16_t *abase = vals + i16 * 16 + kh * 8;
+    const uint32_t a_lane_bytes = (uint32_t)(i16 * 16 + kh * 8) * 2u; // this lane's 16 bytes inside a block
     const f16x8 zero8 = {0, 0, 0, 0, 0, 0, 0, 0};
+    const i32x4 empty_table = {-1, -1, 0, 0};
+
+    // A operands of one chunk: slot k <- the two blocks of op k (lanes 0-31: p1, 32-63: p2).
+    // Loads are unconditional: an empty slot or the missing second block of a single
+    // re-reads a valid block (its data is never used, or is zeroed at use).
+    auto load_a = [&](f16x8 (&dst)[CAP], const i32x4 &tab) {
+#pragma unroll
+        for (int k = 0; k < CAP; k++) {
+            const int p1 = __builtin_amdgcn_readlane(tab[0], k);
+            const int p2 = __builtin_amdgcn_readlane(tab[1], k);
+            // empty slot: every lane reads the first 16 bytes of vals (one cache line)
+            const uint32_t b1 = p1 < 0 ? 0u : (uint32_t)p1 * 512u;
+            const uint32_t b2 = p2 < 0 ? b1 : (uint32_t)p2 * 512u;
+            const uint32_t lo = p1 < 0 ? 0u : a_lane_bytes;
+            const uint32_t off = (sel ? b2 : b1) + lo; // nnzb * 512 < 2^32 is checked by the plan
+            dst[k] = *reinterpret_cast<const f16x8 *>(reinterpret_cast<const char *>(vals) + off);
+        }
+    };
+
+    i32x4 tab_cur = empty_table, tab_nxt = empty_table, tab_nx2 = empty_table;
+    f16x8 a_cur[CAP], a_nxt[CAP];
+#pragma unroll
+    for (int k = 0; k < CAP; k++) { a_cur[k] = zero8; a_nxt[k] = zero8; }
 
     int stage = 0;
-    if (c_begin < c_end) fill_issue(lds, B, chunk_ids[c_begin], n0, N, K, wave, lane);
+    if (c_begin < c_end) {
+        const int last = c_end - 1;
+        tab_cur = load_op_table(ops, c_begin, wave, lane);
+        tab_nxt = load_op_table(ops, c_begin + 1 < last ? c_begin + 1 : last, wave, lane);
+        fill_issue(lds, B, chunk_ids[c_begin] & ~SWEEP_CONT_FLAG, n0, N, K, wave, lane);
+        load_a(a_cur, tab_cur);
+    }
     __builtin_amdgcn_s_waitcnt(0x0f70); // vmcnt(0): the copies of this wavefront have landed
     __syncthreads();
 
     for (int ci = c_begin; ci < c_end; ci++) {
-        // ops of this wavefront in this chunk, grouped by local block row r:
-        // [op_ptr[base + r], op_ptr[base + r + 1])
-        const int base = (ci * W + wave) * RW;
-        const int o_first = op_ptr[base], o_last = op_ptr[base + RW];
-        SweepOp op = {0, -1, 0, 0};
-        f16x8 a = zero8;
-        if (o_first < o_last) { // A operand of the first op: issued ahead of the B copies
-            op = ops[o_first];
-            const int p = sel ? op.p2 : op.p1;
-            a = p >= 0 ? *reinterpret_cast<const f16x8 *>(abase + (long)p * 256) : zero8;
+        // ---- issue everything chunk ci+1 (and the table of ci+2) needs ----
+        // Past the end the last record is simply loaded again: no branches around loads.
+        const int last = c_end - 1;
+        tab_nx2 = load_op_table(ops, ci + 2 < last ? ci + 2 : last, wave, lane);
+#ifndef SMAT_EXP_NO_A
+        load_a(a_nxt, tab_nxt);
+#endif
+        // A record that continues the chunk of the previous record (its ops did not
+        // fit one table) has bit 30 set: no B copy, the LDS stage stays.
+        int next_chunk = 0;
+        bool next_is_new = false;
+        if (ci + 1 < c_end) {
+            next_chunk = chunk_ids[ci + 1];
+            next_is_new = !(next_chunk & SWEEP_CONT_FLAG);
+#ifndef SMAT_EXP_NO_FILL
+            if (next_is_new)
+                fill_issue(lds + (stage ^ 1) * STAGE_BYTES, B, next_chunk, n0, N, K, wave, lane);
+#endif
         }
-        const bool more = ci + 1 < c_end;
-        if (more) fill_issue(lds + (stage ^ 1) * STAGE_BYTES, B, chunk_ids[ci + 1], n0, N, K, wave, lane);
 
+        // ---- MFMA work of chunk ci: registers and LDS only ----
         const unsigned char *cur = lds + stage * STAGE_BYTES + rd_base;
 #pragma unroll
-        for (int r = 0; r < RW; r++) {
-            const int o_end = op_ptr[base + r + 1];
-            for (int o = op_ptr[base + r]; o < o_end; o++) {
-                SweepOp opn = {0, -1, 0, 0};
-                f16x8 an = zero8;
-                if (o + 1 < o_last) { // next op of this wavefront (possibly of the next row)
-                    opn = ops[o + 1];
-                    const int p = sel ? opn.p2 : opn.p1;
-                    an = p >= 0 ? *reinterpret_cast<const f16x8 *>(abase + (long)p * 256) : zero8;
-                }
-                const int s = sel ? ((op.meta >> 16) & 0xff) : ((op.meta >> 8) & 0xff);
-                const int swz = (s >> 3) * (NT * ROW_BYTES) + (((((s & 7) << 1) | kh) ^ i16) << 4);
-                const unsigned char *bp = cur + swz;
+        for (int k = 0; k < CAP; k++) {
+            // slot k belongs to block row k / CAPR of this wavefront: the accumulator
+            // registers of every slot are fixed at compile time
+            constexpr int CAPR = CAP / RW;
+            const int p1 = __builtin_amdgcn_readlane(tab_cur[0], k);
+#ifdef SMAT_EXP_NO_MFMA
+            if (p1 == -12345) {
+#else
+            if (p1 >= 0) {
+#endif
+                // meta = LDS byte offset of the slab of p1 | that of p2 << 16 (without the
+                // per-lane XOR): slab group * NT * 256 + (slab % 8) * 32
+                const uint32_t meta = (uint32_t)__builtin_amdgcn_readlane(tab_cur[2], k);
+                const uint32_t soff = sel ? (meta >> 16) : (meta & 0xffffu);
+                const unsigned char *bp = cur + (soff ^ lane_xor);
+                f16x8 av = a_cur[k];
+                if (__builtin_amdgcn_readlane(tab_cur[1], k) < 0) // single: no second block
+                    av = sel ? zero8 : av;
+#ifdef SMAT_EXP_B8
+                f16x8 b[TN];
+#pragma unroll
+                for (int t = 0; t < TN; t++)
+                    b[t] = *reinterpret_cast<const f16x8 *>(bp + (64 * (t / 4) + 4 * (t % 4)) * ROW_BYTES);
+#pragma unroll
+                for (int t = 0; t < TN; t++)
+                    acc[k / CAPR][t] = __builtin_amdgcn_mfma_f32_16x16x32_f16(b[t], av, acc[k / CAPR][t], 0, 0, 0);
+#else
 #pragma unroll
                 for (int u = 0; u < TN / 4; u++) {
                     f16x8 b[4];
 #pragma unroll
                     for (int tt = 0; tt < 4; tt++)
+#ifdef SMAT_EXP_NO_LDSREAD
+                        b[tt] = a_cur[(k + tt + u) % CAP];
+#else
                         b[tt] = *reinterpret_cast<const f16x8 *>(bp + (64 * u + 4 * tt) * ROW_BYTES);
+#endif
 #pragma unroll
                     for (int tt = 0; tt < 4; tt++)
-                        acc[r][u * 4 + tt] = __builtin_amdgcn_mfma_f32_16x16x32_f16(
-                            b[tt], a, acc[r][u * 4 + tt], 0, 0, 0);
+                        acc[k / CAPR][u * 4 + tt] = __builtin_amdgcn_mfma_f32_16x16x32_f16(
+                            b[tt], av, acc[k / CAPR][u * 4 + tt], 0, 0, 0);
                 }
-                op = opn;
-                a = an;
+#ifndef SMAT_EXP_NO_SCHED
+                // order of the 8 LDS reads and 8 MFMAs of this op: four reads ahead, then one
+                // MFMA per further read, so an MFMA never waits on the read issued just before it
+                __builtin_amdgcn_sched_group_barrier(0x100, 4, 0);
+#pragma unroll
+                for (int q = 0; q < 4; q++) {
+                    __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
+                    __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);
+                }
+                __builtin_amdgcn_sched_group_barrier(0x008, 4, 0);
+#endif
+#endif
             }
         }
-        __builtin_amdgcn_s_waitcnt(0x0f70); // vmcnt(0): this wavefront's copies have landed
-        __syncthreads();
-        stage ^= 1;
-    }
 
+        __builtin_amdgcn_s_waitcnt(0x0f70); // vmcnt(0): next chunk's B, A and table have landed
+#ifndef SMAT_EXP_NO_BARRIER
+        __syncthreads();
+#endif
+        if (next_is_new) stage ^= 1;
+        tab_cur = tab_nxt;
+        tab_nxt = tab_nx2;
+#pragma unroll
+        for (int k = 0; k < CAP; k++) a_cur[k] = a_nxt[k];
+    }
     // Epilogue: acc[r][t][e] = C[(rg*G + wave*RW + r)*16 + i16][n0 + 64*(t/4) + 16*g + 4*(t%4) + e]
 #pragma unroll
     for (int r = 0; r < RW; r++) {
@@ -221,12 +317,12 @@ hipError_t launch_sweep(const SweepArgs &a, hipStream_t st)
     dim3 grid((unsigned)wgs), block(THREADS);
     if (a.c_f32)
         hipLaunchKernelGGL((spmm_sweep_kernel<true>), grid, block, lds_bytes, st, a.vals, a.B, a.C,
-                           a.rg_chunk_ptr, a.chunk_ids, a.op_ptr, a.ops, (int)(a.M / 16), (int)a.N,
-                           (long)a.K, a.n_rg, n_panels);
+                           a.rg_chunk_ptr, a.chunk_ids, a.ops, (int)(a.M / 16), (int)a.N, (long)a.K,
+                           a.n_rg, n_panels);
     else
         hipLaunchKernelGGL((spmm_sweep_kernel<false>), grid, block, lds_bytes, st, a.vals, a.B, a.C,
-                           a.rg_chunk_ptr, a.chunk_ids, a.op_ptr, a.ops, (int)(a.M / 16), (int)a.N,
-                           (long)a.K, a.n_rg, n_panels);
+                           a.rg_chunk_ptr, a.chunk_ids, a.ops, (int)(a.M / 16), (int)a.N, (long)a.K,
+                           a.n_rg, n_panels);
     return hipGetLastError();
 }
 
