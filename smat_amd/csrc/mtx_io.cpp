@@ -127,7 +127,7 @@ extern "C" int smat_mtx_read(const char *path, size_t *M, size_t *K, size_t *nnz
         else if (ok && is_integer) { ok = c.read_long(iv); fv = (double)iv; }
         if (!ok) return set_error(SMAT_ERR_IO, "%s: entry %ld of %ld is missing or malformed", path, i + 1, nz);
         if (a < 1 || a > m || b < 1 || b > n)
-            return set_error(SMAT_ERR_IO, "%s: entry %ld (%ld,%ld) lies outside %ld x %ld", path, i + 1, a, b, m0, n0);
+            return set_error(SMAT_ERR_IO, "%s: entry %ld (%ld,%ld) lies outside the padded %ld x %ld matrix", path, i + 1, a, b, m, n);
         if (sym && b > m)
             return set_error(SMAT_ERR_IO, "%s: symmetric entry %ld cannot be mirrored", path, i + 1);
         ri[i] = (int32_t)(a - 1);

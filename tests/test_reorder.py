@@ -1,0 +1,116 @@
+"""Row reordering: the library against fixtures recorded from the compiled reference
+(tests/golden/reorder/*.npz, made by tests/golden/make_reorder_golden.py) and, when
+oracle/_ref/Matrix_Blocking is present, against the reference program run live."""
+import glob
+import os
+import subprocess
+
+import numpy as np
+import pytest
+
+from smat_amd import generators as gen
+from tests.oracle_lib import ref_binary
+
+HERE = os.path.dirname(os.path.abspath(__file__))
+FIXTURES = sorted(glob.glob(os.path.join(HERE, "golden", "reorder", "*.npz")))
+
+
+def reordered_edges(rows, row_ptr, col_idx, perm):
+    rp = row_ptr.astype(np.int64)
+    cnt = np.diff(rp)[perm]
+    new_rows = np.repeat(np.arange(rows), cnt)
+    new_cols = np.concatenate([col_idx[rp[p]:rp[p + 1]] for p in perm]) if rows else np.zeros(0, np.int64)
+    return new_rows, new_cols
+
+
+def test_fixtures_exist():
+    assert len(FIXTURES) >= 10
+
+
+@pytest.mark.parametrize("path", FIXTURES, ids=[os.path.basename(p)[:-4] for p in FIXTURES])
+def test_grouping_permutation_and_counters_match_reference(smat, path):
+    d = np.load(path)
+    rows, cols = int(d["rows"]), int(d["cols"])
+    for k, (cb, rb, tau) in enumerate(d["params"]):
+        g, perm, stats = smat.reorder_rows(rows, cols, d["row_ptr"], d["col_idx"], int(cb), int(rb),
+                                           float(np.float32(tau)))
+        assert np.array_equal(g, d[f"grouping_{k}"]), (k, "grouping")
+        assert np.array_equal(stats, d[f"stats_{k}"]), (k, "counters")
+        nr, nc = reordered_edges(rows, d["row_ptr"], d["col_idx"], perm)
+        assert np.array_equal(nr, d[f"reordered_rows_{k}"]) and np.array_equal(nc, d[f"reordered_cols_{k}"])
+        assert np.array_equal(np.sort(perm), np.arange(rows))
+
+
+def run_reference(tmp_path, r, c, cb, rb, tau):
+    binary = ref_binary("Matrix_Blocking")
+    el = tmp_path / "case.el"
+    order = np.lexsort((c, r))
+    el.write_text("\n".join(f"{a} {b}" for a, b in zip(r[order].tolist(), c[order].tolist())) + "\n")
+    out = tmp_path / "stats.txt"
+    subprocess.run([binary, "-f", str(el), "-a", "5", "-b", str(cb), "-B", str(rb), "-F", "1", "-t", repr(tau),
+                    "-v", "0", "-o", str(out)], check=True, stdout=subprocess.DEVNULL)
+    fields = (tmp_path / "stats.txt.g").read_text().strip().split(",")
+    return np.array([int(x) for x in fields[1:] if x], dtype=np.int64)
+
+
+@pytest.mark.skipif(ref_binary("Matrix_Blocking") is None, reason="oracle/_ref/Matrix_Blocking not built")
+@pytest.mark.parametrize("seed", range(6))
+def test_live_against_reference_program(smat, tmp_path, seed):
+    rng = np.random.default_rng(seed)
+    rows, cols = int(rng.integers(50, 1500)), int(rng.integers(50, 3000))
+    nnz = int(rows * rng.uniform(1, 12))
+    key = np.unique(rng.integers(0, rows, nnz) * cols + rng.integers(0, cols, nnz))
+    r, c = key // cols, key % cols
+    # duplicate some row patterns so merges happen
+    src = rng.integers(0, rows, rows // 3)
+    extra_r, extra_c = [], []
+    for dst_row, s in enumerate(src):
+        m = r == s
+        extra_r.append(np.full(int(m.sum()), (dst_row * 7) % rows))
+        extra_c.append(c[m])
+    key = np.unique(np.concatenate([r] + extra_r) * cols + np.concatenate([c] + extra_c))
+    r, c = key // cols, key % cols
+    if r.max() != rows - 1:
+        rows = int(r.max()) + 1
+    cb, rb, tau = [(16, 16, 0.5), (8, 16, 0.5), (16, 16, 0.2), (5, 4, 0.6), (16, 16, 0.8), (1, 2, 0.5)][seed]
+    want = run_reference(tmp_path, r, c, cb, rb, tau)
+    row_ptr = np.zeros(rows + 1, dtype=np.int64)
+    np.add.at(row_ptr, r + 1, 1)
+    g, perm, _ = smat.reorder_rows(rows, int(c.max()) + 1, np.cumsum(row_ptr), c, cb, rb, float(np.float32(tau)))
+    assert np.array_equal(g, want)
+
+
+def test_two_pass_flow_and_permute(smat):
+    d = gen.stencil27(10)  # 1000 rows -> padded to 1008
+    M = K = 1008
+    rp = np.concatenate([d["row_ptr"], np.full(8, d["row_ptr"][-1])]).astype(np.int32)
+    pr, pc, sr, sc = smat.reorder_csr(M, K, rp, d["col_idx"], 16, 16, 0.5, do_cols=True)
+    assert np.array_equal(np.sort(pr), np.arange(M)) and np.array_equal(np.sort(pc), np.arange(K))
+    assert np.array_equal(pr[1000:], np.arange(1000, M)) and np.array_equal(pc[1000:], np.arange(1000, K))
+    # row pass alone equals the single-pass API on the 1000 real rows
+    g, perm, stats = smat.reorder_rows(1000, 1000, d["row_ptr"], d["col_idx"], 16, 16, 0.5)
+    assert np.array_equal(pr[:1000], perm) and np.array_equal(sr, stats)
+    # permuting keeps every entry: value multiset per (old row, old col) is preserved
+    rp2, ci2, v2 = smat.permute_csr(M, K, rp, d["col_idx"], d["val"], pr, pc)
+    assert rp2[-1] == rp[-1]
+    inv_c = np.empty(K, np.int64)
+    inv_c[pc] = np.arange(K)
+    for new_r in (0, 17, 500, 999):
+        old = pr[new_r]
+        want = sorted(zip(inv_c[d["col_idx"][rp[old]:rp[old + 1]]].tolist(), d["val"][rp[old]:rp[old + 1]].tolist()))
+        got = list(zip(ci2[rp2[new_r]:rp2[new_r + 1]].tolist(), v2[rp2[new_r]:rp2[new_r + 1]].tolist()))
+        assert got == want
+    # the point of the exercise: fewer nonzero blocks than the natural order here? (not guaranteed in general,
+    # so only the bookkeeping is asserted) -- the block count reported by the pass equals the BCSR of its output
+    a_rows_only = smat.csr_to_bcsr(M, K, *smat.permute_csr(M, K, rp, d["col_idx"], d["val"], pr, None))
+    assert a_rows_only.nnzb == sr[2]
+
+
+def test_bad_arguments(smat):
+    with pytest.raises(smat.SmatError):
+        smat.reorder_rows(2, 4, np.array([0, 2, 3]), np.array([3, 1, 0]), 16, 16, 0.5)  # unsorted row
+    with pytest.raises(smat.SmatError):
+        smat.reorder_rows(1, 4, np.array([0, 1]), np.array([0]), 0, 16, 0.5)
+    with pytest.raises(smat.SmatError):
+        smat.permute_csr(16, 16, np.zeros(17, np.int32), np.zeros(0, np.int32), np.zeros(0, np.uint16),
+                         np.zeros(16, np.int64), None)  # not a permutation
