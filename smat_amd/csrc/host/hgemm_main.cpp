@@ -1,0 +1,45 @@
+// `hgemm`: the benchmark binary of the matrix-load -> block -> SpMM -> verify flow.
+// Accepts the flags of the reference binary (src/cuda_hgemm/src/main.cu:22-34):
+//   -filename -n_mult -warmup_iterations -profiling_iterations -sleep_duration
+//   -enable_check -gpu_rank -cpu_procs  (-M -N -K -enable_wmma -enable_mma are
+//   accepted and ignored: they only sized the dense-GEMM leftovers there)
+// and adds: -reorder (row + column clustering before blocking), -tau,
+//   -random_b (seeded uniform[-1,1] B instead of all ones), -use_plan, -kernel.
+#include <thread>
+
+#include "flags.h"
+#include "tester.h"
+
+int main(int argc, char **argv)
+{
+    Flags f(argc, argv);
+    const int gpu = (int)f.num("gpu_rank", 0);
+    SMAT_CHECK(smat_set_device(gpu));
+    char name[256];
+    SMAT_CHECK(smat_device_name(gpu, name, sizeof name));
+    int64_t cus = 0, lds = 0, mem = 0, clk = 0;
+    SMAT_CHECK(smat_device_attr(gpu, &cus, &lds, &mem, &clk));
+    HLOG("%s start with %ld CPU processes on the %d-th GPU: %s", smat_version(),
+         f.num("cpu_procs", (long)std::thread::hardware_concurrency()), gpu, name);
+    HLOG("%lld compute units, %lld KBytes LDS per CU, %.0f MBytes global memory, clock %.0f MHz", (long long)cus,
+         (long long)(lds / 1024), (double)mem / 1048576.0, (double)clk * 1e-3);
+
+    const std::string file = f.str("filename", "");
+    if (file.empty()) { HLOG("usage: hgemm -filename=<matrix.mtx> [-n_mult=<N/8>] [-enable_check] ..."); return 2; }
+    const int n_mult = (int)f.num("n_mult", 1);
+    HLOG("Input .mtx: %s, N_MULT: %d (N = %d)", file.c_str(), n_mult, n_mult * 8);
+    HLOG("Profiling: warmup iterations: %ld, profiling iterations: %ld, sleep duration: %ld ms, enable check: %d",
+         f.num("warmup_iterations", 1), f.num("profiling_iterations", 10), f.num("sleep_duration", 100),
+         (int)f.flag("enable_check", false));
+
+    Tester tester((size_t)f.num("warmup_iterations", 1), (size_t)f.num("profiling_iterations", 10),
+                  (size_t)f.num("sleep_duration", 100), f.flag("enable_check", false), n_mult, file,
+                  f.flag("reorder", false), (float)f.real("tau", 0.5), f.flag("random_b", false),
+                  f.flag("use_plan", true), (int)f.num("kernel", SMAT_KERNEL_AUTO));
+    if (f.flag("use_plan", true))
+        tester.evaluatePlanned("Smat-Plan-Kernel");
+    else
+        tester.evaluateSparse2(mmaCBTKernel, "Mma-CBT-Kernel"); // the drop-in symbol, as in main.cu:99
+    HLOG("Done");
+    return 0;
+}
