@@ -26,6 +26,12 @@ sys.path.insert(0, ROOT)
 PEAK_FP16_TFLOPS = 2500.0  # MI355X dense fp16 MFMA
 PEAK_HBM_GBS = 8000.0      # MI355X HBM3E
 
+# HBM bytes per launch measured with rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE and scaled by a plain
+# device copy of known size (summaries under profiles/): (workload, kernel id) -> bytes
+MEASURED_TRAFFIC = {
+    ("block_pruned_8192_10pct_N4096", 2): 143441 * 1024 * 2.0 + 65851 * 1024 * 1.0,
+}
+
 
 def build_workload(name):
     from smat_amd import generators as gen
@@ -96,6 +102,9 @@ def main():
     ap.add_argument("--kernel", type=int, default=0, help="0 auto, 1 rowwise, 2 sweep")
     ap.add_argument("--no-plan", action="store_true")
     ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--calibration-copy-mib", type=int, default=0,
+                    help="also run one plain device copy of this many MiB (a kernel of known HBM traffic, "
+                         "to scale rocprofv3 FETCH_SIZE / WRITE_SIZE readings)")
     args = ap.parse_args()
     if args.gpus != 1:
         raise SystemExit("bench.py measures one MI355X: run with --gpus 1 (this build has no multi-GPU path)")
@@ -122,6 +131,13 @@ def main():
 
     def step():
         smat_amd.spmm(vals, rp, ci, Bd, Cd, M, N, K, nnzb, plan=plan, kernel=args.kernel)
+
+    if args.calibration_copy_mib:
+        src = torch.ones(args.calibration_copy_mib << 19, dtype=torch.int16, device=dev)
+        dst = torch.empty_like(src)
+        dst.copy_(src)  # reads and writes calibration_copy_mib MiB each
+        torch.cuda.synchronize()
+        del src, dst
 
     for _ in range(args.warmup):
         step()
@@ -158,7 +174,8 @@ def main():
     else:
         roof = {"bound": "hbm", "achieved": round(ach_gbs, 1), "peak": PEAK_HBM_GBS, "unit": "GB/s",
                 "frac": round(ach_gbs / PEAK_HBM_GBS, 4)}
-    roof["traffic"] = None
+    kernel_id = (plan.info()["kernel"] if plan is not None else 1) if args.kernel == 0 else args.kernel
+    roof["traffic"] = MEASURED_TRAFFIC.get((args.workload, kernel_id))
     roof["kernel_ms"] = round(kernel_ms, 5)
     roof["algorithmic_flops"] = flops
     roof["algorithmic_bytes"] = qbytes
