@@ -160,6 +160,7 @@ __global__ __launch_bounds__(THREADS) void spmm_sweep_kernel(
     };
 
     i32x4 tab_cur = empty_table, tab_nxt = empty_table, tab_nx2 = empty_table;
+
     f16x8 a_cur[CAP], a_nxt[CAP];
 #pragma unroll
     for (int k = 0; k < CAP; k++) { a_cur[k] = zero8; a_nxt[k] = zero8; }
