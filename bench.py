@@ -54,6 +54,11 @@ def build_workload(name):
         b = smat_amd.csr_to_bcsr(d["M"], d["K"], d["row_ptr"], d["col_idx"], d["val"])
         A = {"M": b.M, "K": b.K, "b_row_ptr": b.row_ptr, "b_col_idx": b.col_idx, "b_val": b.val, "nnzb": b.nnzb}
         N, bdist, bseed = 256, "normal", 0xB0000002
+    elif name == "rmat_s20_deg16_N128":
+        d = gen.rmat(20, 16)
+        b = smat_amd.csr_to_bcsr(d["M"], d["K"], d["row_ptr"], d["col_idx"], d["val"])
+        A = {"M": b.M, "K": b.K, "b_row_ptr": b.row_ptr, "b_col_idx": b.col_idx, "b_val": b.val, "nnzb": b.nnzb}
+        N, bdist, bseed = 128, "uniform", 0xB0000003
     else:
         raise SystemExit(f"unknown workload {name}")
     B = gen.dense_b(A["K"], N, seed=bseed, dist=bdist)
@@ -99,7 +104,7 @@ def main():
     ap.add_argument("--steps", type=int, default=200)
     ap.add_argument("--warmup", type=int, default=20)
     ap.add_argument("--workload", default="block_pruned_8192_10pct_N4096")
-    ap.add_argument("--kernel", type=int, default=0, help="0 auto, 1 rowwise, 2 sweep")
+    ap.add_argument("--kernel", type=int, default=0, help="0 auto, 1 rowwise, 2 sweep, 3 rowwise reading B in place")
     ap.add_argument("--no-plan", action="store_true")
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--calibration-copy-mib", type=int, default=0,
@@ -175,6 +180,8 @@ def main():
         roof = {"bound": "hbm", "achieved": round(ach_gbs, 1), "peak": PEAK_HBM_GBS, "unit": "GB/s",
                 "frac": round(ach_gbs / PEAK_HBM_GBS, 4)}
     kernel_id = (plan.info()["kernel"] if plan is not None else 1) if args.kernel == 0 else args.kernel
+    if kernel_id == 1 and (plan is None or not plan.info()["b_pack_bytes"]):
+        kernel_id = 3
     roof["traffic"] = MEASURED_TRAFFIC.get((args.workload, kernel_id))
     roof["kernel_ms"] = round(kernel_ms, 5)
     roof["algorithmic_flops"] = flops

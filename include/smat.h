@@ -64,8 +64,11 @@ int smat_spmm_bcsr_f16(const uint16_t *vals, const int32_t *row_ptr, const int32
 #define SMAT_C_F32 1       /* keep the fp32 accumulators                     */
 
 #define SMAT_KERNEL_AUTO 0
-#define SMAT_KERNEL_ROWWISE 1 /* one wavefront per (block-row chunk, N panel), operands straight from L2 */
+#define SMAT_KERNEL_ROWWISE 1 /* one wavefront per (block-row chunk, N panel), operands straight from L2;
+                               * the plan decides whether B is first repacked slab-major into scratch   */
 #define SMAT_KERNEL_SWEEP 2   /* workgroup sweeps K for a group of block rows, B panel staged in LDS      */
+#define SMAT_KERNEL_ROWWISE_DIRECT 3 /* row-wise, B always read in place (plan or launch option)          */
+#define SMAT_KERNEL_ROWWISE_PACKED 4 /* row-wise, B always repacked (needs a plan created with this id) */
 
 typedef struct smat_spmm_opts {
     int32_t b_layout; /* SMAT_B_COL_MAJOR                                   */
@@ -88,8 +91,9 @@ typedef struct smat_plan smat_plan;
 int smat_plan_create(smat_plan **plan, const int32_t *row_ptr_host, const int32_t *col_idx_host,
                      size_t M, size_t K, size_t nnzb, size_t n_hint, const smat_spmm_opts *opts);
 int smat_plan_destroy(smat_plan *plan);
-/* Fills info[0..7]: kernel id, row-wise work items, split block rows, chunk size,
- * workspace bytes, panel width, sweep MFMA ops, sweep (row group, K chunk) records. */
+/* Fills info[0..8]: kernel id, row-wise work items, split block rows, chunk size,
+ * workspace bytes, panel width, sweep MFMA ops, sweep (row group, K chunk) records,
+ * bytes of the slab-major scratch copy of B (0 = B is read in place). */
 int smat_plan_info(const smat_plan *plan, int64_t *info);
 
 /* Same operands as smat_spmm_bcsr_f16; C is uint16_t* or float* per opts->c_dtype.

@@ -34,6 +34,7 @@ struct smat_plan {
     SplitRow *d_split = nullptr;
     float *d_workspace = nullptr;
     size_t workspace_bytes = 0;
+    uint16_t *d_bpack = nullptr; // slab-major copy of B, K * n_cap halves (row-wise kernel, when it pays)
     // sweep kernel work list (present when kernel == SMAT_KERNEL_SWEEP)
     int n_rg = 0, n_records = 0, n_ops = 0;
     int32_t *d_rg_chunk_ptr = nullptr, *d_chunk_ids = nullptr;
@@ -92,9 +93,13 @@ extern "C" int smat_spmm_bcsr_f16_ex(const uint16_t *vals, const int32_t *row_pt
         a.split_rows = plan->d_split; a.n_split_rows = plan->n_split_rows;
         a.workspace = plan->d_workspace;
         a.panel_tiles = plan->panel_tiles;
+        if (plan->d_bpack && N <= plan->n_cap && o.kernel != SMAT_KERNEL_ROWWISE_DIRECT) a.b_packed = plan->d_bpack;
     }
     int kernel = o.kernel;
     if (kernel == SMAT_KERNEL_AUTO) kernel = plan ? plan->kernel : SMAT_KERNEL_ROWWISE;
+    if (kernel == SMAT_KERNEL_ROWWISE_PACKED && !a.b_packed)
+        return set_error(SMAT_ERR_INVALID, "SMAT_KERNEL_ROWWISE_PACKED needs a plan built for it with n_hint >= N");
+    if (kernel == SMAT_KERNEL_ROWWISE_DIRECT || kernel == SMAT_KERNEL_ROWWISE_PACKED) kernel = SMAT_KERNEL_ROWWISE;
     if (kernel != SMAT_KERNEL_ROWWISE && kernel != SMAT_KERNEL_SWEEP)
         return set_error(SMAT_ERR_INVALID, "unknown kernel id %d", kernel);
     hipError_t e;
@@ -152,7 +157,6 @@ extern "C" int smat_plan_create(smat_plan **out, const int32_t *row_ptr_host,
     smat_plan *p = new (std::nothrow) smat_plan();
     if (!p) return set_error(SMAT_ERR_NOMEM, "out of host memory");
     p->M = M; p->K = K; p->nnzb = nnzb; p->n_cap = n_hint;
-    p->panel_tiles = rowwise_panel_tiles(n_hint, 0);
 
     // A block row is split when it is much longer than the average: chunks of
     // `chunk` blocks (even, so block pairs stay aligned with the MFMA K = 32).
@@ -185,6 +189,7 @@ extern "C" int smat_plan_create(smat_plan **out, const int32_t *row_ptr_host,
         items.push_back(WorkItem{(int32_t)i, row_ptr_host[i], row_ptr_host[i + 1], -1});
     }
     p->n_items = (int)items.size();
+    p->panel_tiles = rowwise_panel_tiles(n_hint, 0, items.size());
     p->n_split_rows = (int)split.size();
     p->n_slots = slot;
 
@@ -198,12 +203,24 @@ extern "C" int smat_plan_create(smat_plan **out, const int32_t *row_ptr_host,
         p->workspace_bytes = (size_t)slot * 16 * n_hint * sizeof(float);
         if (e == hipSuccess) e = hipMalloc(&p->d_workspace, p->workspace_bytes);
     }
+    // Row-wise kernel: repacking B slab-major costs a launch plus one read and one write of B
+    // per SpMM (about 3 us + 4*K*N bytes at 4 TB/s) and lets the operand gather, nnzb*16*N*2
+    // bytes, run at about 20 TB/s instead of 7.6 TB/s (measured on the row-wise kernel).
+    {
+        const double gather_bytes = (double)nnzb * 16.0 * (double)n_hint * 2.0;
+        const double gain_us = gather_bytes * (1.0 / 7.6e6 - 1.0 / 20e6);
+        const double cost_us = 3.0 + 4.0 * (double)K * (double)n_hint / 4e6;
+        if (e == hipSuccess && want != SMAT_KERNEL_ROWWISE_DIRECT &&
+            (gain_us > 1.5 * cost_us || want == SMAT_KERNEL_ROWWISE_PACKED))
+            e = hipMalloc(&p->d_bpack, K * n_hint * sizeof(uint16_t));
+    }
     // The sweep kernel pays one pass over the B panel per group of 32 block rows,
-    // whatever the sparsity: worth it only when a few percent of the blocks exist
-    // and N is wide.
+    // whatever the sparsity, and shares each staged slab between the blocks of the group
+    // that sit in that block column: it overtakes the row-wise kernel at about 10% of the
+    // blocks present, with N wide enough for many panels.
     bool sweep = want == SMAT_KERNEL_SWEEP;
-    if (want == SMAT_KERNEL_AUTO && col_idx_host && n_hint >= 128 && mb >= (size_t)SWEEP_G &&
-        (double)nnzb >= 0.02 * (double)mb * (double)kb)
+    if (want == SMAT_KERNEL_AUTO && col_idx_host && n_hint >= 512 && mb >= 2 * (size_t)SWEEP_G &&
+        (double)nnzb >= 0.08 * (double)mb * (double)kb)
         sweep = true;
     if (sweep && nnzb >= (size_t)1 << 23) { // the sweep kernel addresses blocks with 32-bit byte offsets
         if (want == SMAT_KERNEL_SWEEP) {
@@ -304,6 +321,7 @@ extern "C" int smat_plan_destroy(smat_plan *p)
     if (p->d_items) (void)hipFree(p->d_items);
     if (p->d_split) (void)hipFree(p->d_split);
     if (p->d_workspace) (void)hipFree(p->d_workspace);
+    if (p->d_bpack) (void)hipFree(p->d_bpack);
     if (p->d_rg_chunk_ptr) (void)hipFree(p->d_rg_chunk_ptr);
     if (p->d_chunk_ids) (void)hipFree(p->d_chunk_ids);
     if (p->d_ops) (void)hipFree(p->d_ops);
@@ -318,6 +336,7 @@ extern "C" int smat_plan_info(const smat_plan *p, int64_t *info)
     info[4] = (int64_t)p->workspace_bytes;
     info[5] = p->kernel == SMAT_KERNEL_SWEEP ? 16 * SWEEP_TN : 16 * p->panel_tiles;
     info[6] = p->n_ops; info[7] = p->n_records;
+    info[8] = p->d_bpack ? (int64_t)(p->K * p->n_cap * sizeof(uint16_t)) : 0;
     return SMAT_OK;
 }
 

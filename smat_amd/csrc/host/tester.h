@@ -42,7 +42,7 @@ public:
             smat_spmm_opts o = {SMAT_B_COL_MAJOR, SMAT_C_F16, kernel_, 0, nullptr};
             SMAT_CHECK(smat_plan_create(&plan_, A_->hostBcsrRowPtr(), A_->hostBcsrColIdx(), A_->getRow(), A_->getCol(),
                                         A_->getNonzeroblocks(), N, &o));
-            int64_t info[8];
+            int64_t info[9];
             SMAT_CHECK(smat_plan_info(plan_, info));
             HLOG("Plan: kernel %lld, %lld work items, %lld split block rows, workspace %lld bytes, %lld sweep ops",
                  (long long)info[0], (long long)info[1], (long long)info[2], (long long)info[4], (long long)info[6]);

@@ -37,6 +37,7 @@ struct SpmmArgs {
     const SplitRow *split_rows; // device
     int n_split_rows;
     float *workspace; // device, n_slots * 16 * N floats
+    uint16_t *b_packed; // device scratch of K * N halves, or nullptr: read the column-major B directly
 };
 
 // One MFMA worth of work in the sweep kernel: two blocks of the same block row
@@ -75,7 +76,7 @@ struct SweepArgs {
     int n_rg;
 };
 
-int rowwise_panel_tiles(size_t N, int requested);
+int rowwise_panel_tiles(size_t N, int requested, size_t n_items);
 hipError_t launch_sweep(const SweepArgs &a, hipStream_t st);
 hipError_t launch_rowwise(const SpmmArgs &a, hipStream_t st);
 

@@ -21,6 +21,12 @@
 
 #include "spmm_kernels.h"
 
+#define SMAT_ORDER_FENCE()                      \
+    do {                                        \
+        asm volatile("" ::: "memory");          \
+        __builtin_amdgcn_sched_barrier(0);      \
+    } while (0)
+
 namespace smat {
 
 typedef _Float16 f16x8 __attribute__((ext_vector_type(8)));
@@ -59,8 +65,15 @@ __device__ __forceinline__ int ncol_of(int t, int i)
 // ids are dealt round-robin to the 8 XCDs by the dispatcher; the remap below
 // gives each XCD a contiguous eighth of the (panel-major) item space so that an
 // XCD's private L2 holds few distinct B panels.
-template <int TN, bool C_F32>
-__global__ __launch_bounds__(256) void spmm_rowwise_kernel(
+// amdgpu_waves_per_eu(1, 4): at most 4 wavefronts per SIMD are asked for, which leaves the
+// compiler 128 registers; with the default target of 8 it squeezes the kernel into 64 and
+// gets there by loading each operand right before its MFMA, one memory latency apiece.
+//
+// PACKED: B is the slab-major copy made by pack_b_kernel, Bp[(bc/16 * N + n) * 16 + k % 16]:
+// the 16 x 16 operand of one (block column, n-tile) is 512 contiguous bytes and a
+// wavefront load touches 8 full cache lines instead of 32 quarter-used ones.
+template <int TN, bool C_F32, bool PACKED>
+__global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 4))) void spmm_rowwise_kernel(
     const uint16_t *__restrict__ vals, const int32_t *__restrict__ row_ptr,
     const int32_t *__restrict__ col_idx, const uint16_t *__restrict__ B, void *__restrict__ Cout,
     float *__restrict__ workspace, const WorkItem *__restrict__ items, int n_items, int N, long K,
@@ -100,35 +113,69 @@ __global__ __launch_bounds__(256) void spmm_rowwise_kernel(
 
     f32x4 acc[TN];
     long boff[TN];
-    bool nok[TN];
 #pragma unroll
     for (int t = 0; t < TN; t++) {
         acc[t] = (f32x4){0.f, 0.f, 0.f, 0.f};
-        int n = n0 + ncol_of<TN>(t, i16);
-        nok[t] = n < N;
-        boff[t] = (long)(nok[t] ? n : 0) * K + kh * 8;
+        // columns past N read column 0 instead: what they produce is never stored
+        const int n = n0 + ncol_of<TN>(t, i16);
+        boff[t] = PACKED ? (long)(n < N ? n : 0) * 16 + kh * 8 : (long)(n < N ? n : 0) * K + kh * 8;
     }
     const uint16_t *abase = vals + i16 * 16 + kh * 8;
+    const f16x8 zero8 = zero_f16x8();
 
+    // Every load below is unconditional (indices are clamped instead of branching): loads
+    // inside branches cannot be counted by the compiler's vmcnt bookkeeping, which then
+    // waits for everything in flight and serialises load and MFMA phases.
+    // Two register sets: the operands of pair j+1 are in flight while pair j is multiplied.
     for (int pb = p0; pb < p1; pb += 64) {
         const int cnt = (p1 - pb) < 64 ? (p1 - pb) : 64;
+        const int npair = (cnt + 1) >> 1;
         // one coalesced load of up to 64 column indices, then lane broadcasts
-        const int myc = (lane < cnt) ? col_idx[pb + lane] : 0;
-        for (int j = 0; j < cnt; j += 2) {
-            const int c0 = __builtin_amdgcn_readlane(myc, j);
-            const int c1 = __builtin_amdgcn_readlane(myc, (j + 1) & 63);
-            const bool valid = (sel == 0) || (j + 1 < cnt);
+        const int myc = col_idx[pb + (lane < cnt ? lane : cnt - 1)];
+
+        auto issue = [&](int j, f16x8 &a, f16x8 (&b)[TN]) {
+            const int jj = j < npair ? j : npair - 1; // past the end: reload the last pair (unused)
+            const int second = (2 * jj + 1 < cnt) ? 2 * jj + 1 : 2 * jj; // a single block pairs with itself
+            const int c0 = __builtin_amdgcn_readlane(myc, 2 * jj);
+            const int c1 = __builtin_amdgcn_readlane(myc, second);
             const int bc = sel ? c1 : c0;
-            const long pp = (long)pb + j + sel;
-            f16x8 a = valid ? load_f16x8(abase + pp * 256) : zero_f16x8();
-            f16x8 b[TN];
+            const long pp = (long)pb + (sel ? second : 2 * jj);
+#ifdef SMAT_EXP_NT_A
+            a = __builtin_nontemporal_load(reinterpret_cast<const f16x8 *>(abase + pp * 256));
+#else
+            a = load_f16x8(abase + pp * 256);
+#endif
+            // column-major: + first column of the block; packed: + slab of the block column
+            const long boffs = PACKED ? (long)bc * N : (long)bc;
 #pragma unroll
-            for (int t = 0; t < TN; t++)
-                b[t] = (valid && nok[t]) ? load_f16x8(B + boff[t] + bc) : zero_f16x8();
+            for (int t = 0; t < TN; t++) b[t] = load_f16x8(B + boff[t] + boffs);
+        };
+        auto multiply = [&](int j, f16x8 a, const f16x8 (&b)[TN]) {
+            if (2 * j + 1 >= cnt) a = sel ? zero8 : a; // single block: the upper K half contributes nothing
 #pragma unroll
             for (int t = 0; t < TN; t++)
                 acc[t] = __builtin_amdgcn_mfma_f32_16x16x32_f16(b[t], a, acc[t], 0, 0, 0);
+        };
+
+        // The main loop multiplies two pairs per trip with no branch around either of them:
+        // a multiply inside a branch drags its loads into the branch with it (they sink to
+        // their only use) and the prefetch distance collapses.  The fences pin the issue
+        // order against the scheduler.
+        f16x8 a0, a1, b0[TN], b1[TN];
+        issue(0, a0, b0);
+        SMAT_ORDER_FENCE();
+        int j = 0;
+        for (; j + 2 <= npair; j += 2) {
+            issue(j + 1, a1, b1);
+            SMAT_ORDER_FENCE();
+            multiply(j, a0, b0);
+            SMAT_ORDER_FENCE();
+            issue(j + 2, a0, b0); // past the end this reloads the last pair, unused
+            SMAT_ORDER_FENCE();
+            multiply(j + 1, a1, b1);
+            SMAT_ORDER_FENCE();
         }
+        if (j < npair) multiply(j, a0, b0); // odd number of pairs: the last one is already in set 0
     }
 
     // Epilogue.  acc[t][r] = C[br*16 + i16][n0 + ncol_of(t, 4*g + r)].
@@ -199,6 +246,35 @@ __global__ __launch_bounds__(256) void spmm_reduce_kernel(const float *__restric
     }
 }
 
+// Column-major B (B[n*K + k]) -> slab-major Bp[(k/16 * N + n) * 16 + k % 16].
+// One workgroup moves a tile of 64 n x 64 k through LDS: reads are 128-byte runs along k,
+// writes are 2 KiB runs (64 n x 32 B) per block column.
+__global__ __launch_bounds__(256) void pack_b_kernel(const uint16_t *__restrict__ B,
+                                                     uint16_t *__restrict__ Bp, int N, long K)
+{
+    __shared__ __align__(16) unsigned char tile[8192];
+    const int t = threadIdx.x;
+    const long k0 = (long)blockIdx.x * 64;
+    const int n0 = blockIdx.y * 64;
+#pragma unroll
+    for (int i = 0; i < 2; i++) {
+        const int idx = i * 256 + t;
+        const int nl = idx >> 3, seg = idx & 7; // seg: 8 k (16 bytes) along k
+        f16x8 v = zero_f16x8();
+        if (n0 + nl < N && k0 + seg * 8 < K) v = load_f16x8(B + (long)(n0 + nl) * K + k0 + seg * 8);
+        *reinterpret_cast<f16x8 *>(tile + ((seg >> 1) * 64 + nl) * 32 + (seg & 1) * 16) = v;
+    }
+    __syncthreads();
+#pragma unroll
+    for (int i = 0; i < 2; i++) {
+        const int idx = i * 256 + t;
+        const int bcl = idx >> 7, nl = (idx & 127) >> 1, half = idx & 1;
+        if (n0 + nl < N && k0 + bcl * 16 < K)
+            *reinterpret_cast<f16x8 *>(Bp + ((k0 / 16 + bcl) * N + n0 + nl) * 16 + half * 8) =
+                *reinterpret_cast<const f16x8 *>(tile + (size_t)idx * 16);
+    }
+}
+
 template <int TN>
 static hipError_t launch_rowwise_tn(const SpmmArgs &a, hipStream_t st)
 {
@@ -210,21 +286,28 @@ static hipError_t launch_rowwise_tn(const SpmmArgs &a, hipStream_t st)
     if (wgs == 0) return hipSuccess;
     if (wgs > 0x7fffffffL) return hipErrorInvalidValue;
     dim3 grid((unsigned)wgs), block(256);
-    if (a.c_f32)
-        hipLaunchKernelGGL((spmm_rowwise_kernel<TN, true>), grid, block, 0, st, a.vals, a.row_ptr,
-                           a.col_idx, a.B, a.C, a.workspace, a.items, a.n_items, (int)a.N,
-                           (long)a.K, n_panels);
-    else
-        hipLaunchKernelGGL((spmm_rowwise_kernel<TN, false>), grid, block, 0, st, a.vals, a.row_ptr,
-                           a.col_idx, a.B, a.C, a.workspace, a.items, a.n_items, (int)a.N,
-                           (long)a.K, n_panels);
+#define SMAT_LAUNCH_ROWWISE(F32, PK)                                                              \
+    hipLaunchKernelGGL((spmm_rowwise_kernel<TN, F32, PK>), grid, block, 0, st, a.vals, a.row_ptr, \
+                       a.col_idx, a.b_packed ? a.b_packed : a.B, a.C, a.workspace, a.items,       \
+                       a.n_items, (int)a.N, (long)a.K, n_panels)
+    if (a.b_packed) {
+        if (a.c_f32) SMAT_LAUNCH_ROWWISE(true, true);
+        else SMAT_LAUNCH_ROWWISE(false, true);
+    } else {
+        if (a.c_f32) SMAT_LAUNCH_ROWWISE(true, false);
+        else SMAT_LAUNCH_ROWWISE(false, false);
+    }
+#undef SMAT_LAUNCH_ROWWISE
     return hipGetLastError();
 }
 
-int rowwise_panel_tiles(size_t N, int requested)
+int rowwise_panel_tiles(size_t N, int requested, size_t n_items)
 {
     if (requested == 1 || requested == 2 || requested == 4 || requested == 8) return requested;
     if (N >= 512) return 8;
+    // 128-column panels read every block of A once per 128 instead of 64 columns of C: take
+    // them as soon as the work list alone fills the chip (256 CUs x 16 wavefronts)
+    if (N >= 128 && n_items * (N / 128) >= 4096) return 8;
     if (N >= 64) return 4;
     if (N >= 32) return 2;
     return 1;
@@ -233,7 +316,13 @@ int rowwise_panel_tiles(size_t N, int requested)
 hipError_t launch_rowwise(const SpmmArgs &a, hipStream_t st)
 {
     hipError_t e;
-    switch (rowwise_panel_tiles(a.N, a.panel_tiles)) {
+    if (a.b_packed) {
+        dim3 grid((unsigned)((a.K + 63) / 64), (unsigned)((a.N + 63) / 64));
+        hipLaunchKernelGGL(pack_b_kernel, grid, dim3(256), 0, st, a.B, a.b_packed, (int)a.N, (long)a.K);
+        e = hipGetLastError();
+        if (e != hipSuccess) return e;
+    }
+    switch (rowwise_panel_tiles(a.N, a.panel_tiles, (size_t)a.n_items)) {
     case 8: e = launch_rowwise_tn<8>(a, st); break;
     case 4: e = launch_rowwise_tn<4>(a, st); break;
     case 2: e = launch_rowwise_tn<2>(a, st); break;

@@ -11,7 +11,7 @@ import numpy as np
 from ._lib import SpmmOpts, check, lib
 
 BS = 16
-KERNEL_AUTO, KERNEL_ROWWISE, KERNEL_SWEEP = 0, 1, 2
+KERNEL_AUTO, KERNEL_ROWWISE, KERNEL_SWEEP, KERNEL_ROWWISE_DIRECT, KERNEL_ROWWISE_PACKED = 0, 1, 2, 3, 4
 C_F16, C_F32 = 0, 1
 
 
@@ -131,9 +131,10 @@ class Plan:
         return self._h
 
     def info(self):
-        out = (C.c_int64 * 8)()
+        out = (C.c_int64 * 9)()
         check(lib.smat_plan_info(self._h, out))
-        keys = ("kernel", "items", "split_rows", "chunk", "workspace_bytes", "panel", "sweep_ops", "sweep_records")
+        keys = ("kernel", "items", "split_rows", "chunk", "workspace_bytes", "panel", "sweep_ops", "sweep_records",
+                "b_pack_bytes")
         return dict(zip(keys, out))
 
     def close(self):

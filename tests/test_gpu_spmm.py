@@ -97,6 +97,40 @@ def test_random_bcsr_all_panel_widths(smat, cuda, oracle, N):
     assert np.array_equal(C32.astype(np.float16).view(np.uint16), C)
 
 
+@pytest.mark.parametrize("mb,kb,density,N,n_hint", [
+    (40, 128, 0.30, 256, 256),
+    (24, 160, 0.25, 264, 264),    # N not a multiple of the 64-column repack tile
+    (33, 130, 0.20, 200, 512),    # plan built for a wider N than the launch uses
+    (64, 256, 0.10, 1032, 1032),  # several N panels, ragged last one
+])
+def test_repacked_b_rowwise_is_bit_identical_to_direct(smat, cuda, oracle, mb, kb, density, N, n_hint):
+    """The slab-major scratch copy of B changes addresses only: same products, same order."""
+    import torch
+    A = gen.random_bcsr(mb, kb, density, seed=mb * 7 + kb)
+    B = gen.dense_b(A["K"], N, seed=N + 3, dist="normal")
+    M, K, nnzb = A["M"], A["K"], int(A["b_col_idx"].shape[0])
+    vals, Bd = to_dev(torch, A["b_val"], cuda), to_dev(torch, B, cuda)
+    rp, ci = to_dev(torch, A["b_row_ptr"].astype(np.int32), cuda), to_dev(torch, A["b_col_idx"].astype(np.int32), cuda)
+    out = {}
+    for kernel in (4, 3):  # always repacked, never repacked
+        p = smat.Plan(A["b_row_ptr"], M, K, nnzb, n_hint, col_idx_host=A["b_col_idx"], kernel=kernel)
+        assert (p.info()["b_pack_bytes"] > 0) == (kernel == 4)
+        for c_f32 in (False, True):
+            C = torch.full((M, N), float("nan"), dtype=torch.float32, device=cuda) if c_f32 else \
+                torch.full((M, N), 0x7E00, dtype=torch.int16, device=cuda)
+            smat.spmm(vals, rp, ci, Bd, C, M, N, K, nnzb, plan=p, c_f32=c_f32, kernel=kernel)
+            torch.cuda.synchronize()
+            out[kernel, c_f32] = C.cpu().numpy()
+        p.close()
+    assert np.array_equal(out[4, False], out[3, False])
+    assert np.array_equal(out[4, True].view(np.uint32), out[3, True].view(np.uint32))
+    ref = oracle_ref(oracle, A, B, N)
+    assert oracle.compare(out[4, False].view(np.uint16), ref)[0] <= TOL_F16
+    assert rel_err_f32(out[4, True], ref) <= TOL_F32
+    assert not np.array_equal(B, 0)  # B itself is left untouched by the repack
+    assert np.array_equal(Bd.cpu().numpy().view(np.uint16), B)
+
+
 def test_drop_in_entry_matches_options_entry(smat, cuda, oracle):
     A = gen.random_bcsr(20, 20, 0.2, seed=5)
     N = 96
