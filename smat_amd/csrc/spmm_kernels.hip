@@ -140,11 +140,7 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 4))) voi
             const int c1 = __builtin_amdgcn_readlane(myc, second);
             const int bc = sel ? c1 : c0;
             const long pp = (long)pb + (sel ? second : 2 * jj);
-#ifdef SMAT_EXP_NT_A
-            a = __builtin_nontemporal_load(reinterpret_cast<const f16x8 *>(abase + pp * 256));
-#else
             a = load_f16x8(abase + pp * 256);
-#endif
             // column-major: + first column of the block; packed: + slab of the block column
             const long boffs = PACKED ? (long)bc * N : (long)bc;
 #pragma unroll
@@ -305,9 +301,10 @@ int rowwise_panel_tiles(size_t N, int requested, size_t n_items)
 {
     if (requested == 1 || requested == 2 || requested == 4 || requested == 8) return requested;
     if (N >= 512) return 8;
-    // 128-column panels read every block of A once per 128 instead of 64 columns of C: take
-    // them as soon as the work list alone fills the chip (256 CUs x 16 wavefronts)
-    if (N >= 128 && n_items * (N / 128) >= 4096) return 8;
+    // Below that, 64-column panels: measured faster than 128-column ones even where the work
+    // list alone fills the chip (R-MAT scale 20, N = 128: 13.8 ms against 18.2 ms), more
+    // wavefronts in flight outweighing the second pass over A.
+    (void)n_items;
     if (N >= 64) return 4;
     if (N >= 32) return 2;
     return 1;
