@@ -17,15 +17,14 @@
 //    (so the accumulator registers of every slot are known at compile time):
 //    pairs of blocks of one block row inside the chunk feed one
 //    v_mfma_f32_16x16x32_f16 (K = 32 = 2 blocks).  A chunk whose ops do not fit
-//    the table continues in a following record that reuses the resident B stage.  A operands are 512-byte coalesced global reads
-//    straight into MFMA layout.
+//    the table continues in a following record that reuses the resident B stage.
+//    A operands are 512-byte coalesced global reads straight into MFMA layout.
 //  * Software pipeline over chunks, everything for chunk c+1 is issued before the
 //    MFMA work of chunk c starts and is only waited for after it: the op table of
 //    chunk c+2, the A operands of chunk c+1 (into a second set of registers) and
 //    the B panel of chunk c+1 (global -> LDS asynchronously with
 //    global_load_lds_dwordx4, no staging registers, into the other LDS stage).
 //    The MFMA loop itself touches only registers and LDS.  One barrier per chunk.
-
 //
 // Same operand semantics as the reference launcher
 // (src/cuda_hgemm/src/mma/mmaCBT.cu:83-88).
@@ -181,9 +180,7 @@ __global__ __launch_bounds__(THREADS) void spmm_sweep_kernel(
         // Past the end the last record is simply loaded again: no branches around loads.
         const int last = c_end - 1;
         tab_nx2 = load_op_table(ops, ci + 2 < last ? ci + 2 : last, wave, lane);
-#ifndef SMAT_EXP_NO_A
         load_a(a_nxt, tab_nxt);
-#endif
         // A record that continues the chunk of the previous record (its ops did not
         // fit one table) has bit 30 set: no B copy, the LDS stage stays.
         int next_chunk = 0;
@@ -191,10 +188,8 @@ __global__ __launch_bounds__(THREADS) void spmm_sweep_kernel(
         if (ci + 1 < c_end) {
             next_chunk = chunk_ids[ci + 1];
             next_is_new = !(next_chunk & SWEEP_CONT_FLAG);
-#ifndef SMAT_EXP_NO_FILL
             if (next_is_new)
                 fill_issue(lds + (stage ^ 1) * STAGE_BYTES, B, next_chunk, n0, N, K, wave, lane);
-#endif
         }
 
         // ---- MFMA work of chunk ci: registers and LDS only ----
@@ -205,11 +200,7 @@ __global__ __launch_bounds__(THREADS) void spmm_sweep_kernel(
             // registers of every slot are fixed at compile time
             constexpr int CAPR = CAP / RW;
             const int p1 = __builtin_amdgcn_readlane(tab_cur[0], k);
-#ifdef SMAT_EXP_NO_MFMA
-            if (p1 == -12345) {
-#else
             if (p1 >= 0) {
-#endif
                 // meta = LDS byte offset of the slab of p1 | that of p2 << 16 (without the
                 // per-lane XOR): slab group * NT * 256 + (slab % 8) * 32
                 const uint32_t meta = (uint32_t)__builtin_amdgcn_readlane(tab_cur[2], k);
@@ -218,31 +209,17 @@ __global__ __launch_bounds__(THREADS) void spmm_sweep_kernel(
                 f16x8 av = a_cur[k];
                 if (__builtin_amdgcn_readlane(tab_cur[1], k) < 0) // single: no second block
                     av = sel ? zero8 : av;
-#ifdef SMAT_EXP_B8
-                f16x8 b[TN];
-#pragma unroll
-                for (int t = 0; t < TN; t++)
-                    b[t] = *reinterpret_cast<const f16x8 *>(bp + (64 * (t / 4) + 4 * (t % 4)) * ROW_BYTES);
-#pragma unroll
-                for (int t = 0; t < TN; t++)
-                    acc[k / CAPR][t] = __builtin_amdgcn_mfma_f32_16x16x32_f16(b[t], av, acc[k / CAPR][t], 0, 0, 0);
-#else
 #pragma unroll
                 for (int u = 0; u < TN / 4; u++) {
                     f16x8 b[4];
 #pragma unroll
                     for (int tt = 0; tt < 4; tt++)
-#ifdef SMAT_EXP_NO_LDSREAD
-                        b[tt] = a_cur[(k + tt + u) % CAP];
-#else
                         b[tt] = *reinterpret_cast<const f16x8 *>(bp + (64 * u + 4 * tt) * ROW_BYTES);
-#endif
 #pragma unroll
                     for (int tt = 0; tt < 4; tt++)
                         acc[k / CAPR][u * 4 + tt] = __builtin_amdgcn_mfma_f32_16x16x32_f16(
                             b[tt], av, acc[k / CAPR][u * 4 + tt], 0, 0, 0);
                 }
-#ifndef SMAT_EXP_NO_SCHED
                 // order of the 8 LDS reads and 8 MFMAs of this op: four reads ahead, then one
                 // MFMA per further read, so an MFMA never waits on the read issued just before it
                 __builtin_amdgcn_sched_group_barrier(0x100, 4, 0);
@@ -252,15 +229,11 @@ __global__ __launch_bounds__(THREADS) void spmm_sweep_kernel(
                     __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);
                 }
                 __builtin_amdgcn_sched_group_barrier(0x008, 4, 0);
-#endif
-#endif
             }
         }
 
         __builtin_amdgcn_s_waitcnt(0x0f70); // vmcnt(0): next chunk's B, A and table have landed
-#ifndef SMAT_EXP_NO_BARRIER
         __syncthreads();
-#endif
         if (next_is_new) stage ^= 1;
         tab_cur = tab_nxt;
         tab_nxt = tab_nx2;
