@@ -98,6 +98,52 @@ def cpu_baseline(A, B, N, target_s=12.0):
                       f"OpenMP over block rows, includes widening B to fp32"}
 
 
+def cpu_baseline_reference(A, B, N, target_s=10.0):
+    """The reference's own serial CSR::multiply (preprocess/src/general/csr.cpp:47-63), compiled from the
+    reference tree into oracle/_ref/, on a leading principal submatrix of A (it indexes B with A's row
+    count, so the sample has to be square) and the matching rows of B, all N columns."""
+    import subprocess
+    import tempfile
+    from tests.oracle_lib import ref_binary
+    from smat_amd import generators as gen
+    exe = ref_binary("ref_csr_multiply")
+    if exe is None:
+        return None
+    mb = min(A["M"], A["K"]) // 16
+    K = A["K"]
+    Bf = B.view(np.float16).reshape(N, K)  # column-major: row n of this view is column n of B
+
+    def run(rb):
+        rp, ci = A["b_row_ptr"], A["b_col_idx"]
+        keep = np.concatenate([np.arange(rp[r], rp[r + 1])[ci[rp[r]:rp[r + 1]] < 16 * rb] for r in range(rb)]) \
+            if rb else np.zeros(0, np.int64)
+        sub_rp = np.zeros(rb + 1, np.int32)
+        for r in range(rb):
+            sub_rp[r + 1] = sub_rp[r] + int((ci[rp[r]:rp[r + 1]] < 16 * rb).sum())
+        sub = {"M": 16 * rb, "b_row_ptr": sub_rp, "b_col_idx": ci[keep], "b_val": A["b_val"].reshape(-1, 256)[keep].ravel()}
+        crp, cci, cv = gen.bcsr_to_csr(sub["M"], sub["b_row_ptr"], sub["b_col_idx"], sub["b_val"])
+        nz = cv != 0
+        vals = cv.view(np.float16).astype(np.float64)
+        rows = np.repeat(np.arange(sub["M"]), np.diff(crp))
+        with tempfile.TemporaryDirectory() as d:
+            with open(os.path.join(d, "a.el"), "w") as f:
+                f.write("".join(f"{r} {c} {v:.10g}\n" for r, c, v in zip(rows[nz], cci[nz], vals[nz])))
+                f.write(f"{sub['M'] - 1} {sub['M'] - 1} 0\n")  # pins rows = cols = 16 * rb in the reference reader
+            np.ascontiguousarray(Bf[:, :16 * rb]).astype(np.float32).tofile(os.path.join(d, "b.f32"))
+            out = subprocess.run([exe, os.path.join(d, "a.el"), os.path.join(d, "b.f32"), str(N), "1"],
+                                 check=True, capture_output=True, text=True).stdout.split()
+        return float(out[3]), int(nz.sum())
+
+    rb = min(mb, 32)
+    t, nnz = run(rb)
+    while t < target_s / 4 and rb < mb:  # nnz of a principal submatrix grows with rb squared
+        rb = int(min(mb, max(rb + 1, rb * min(4.0, (target_s / max(t, 1e-3)) ** 0.5))))
+        t, nnz = run(rb)
+    return {"value": round(2.0 * nnz * N / t / 1e9, 3), "unit": "GFLOP/s", "cores": 1, "kind": "reference",
+            "sample": f"leading {16 * rb} x {16 * rb} submatrix of A ({nnz} nonzeros) times the matching {16 * rb} x {N} "
+                      f"rows of B, {t:.2f} s, reference CSR::multiply (serial, fp32), flops = 2*nnz*N"}
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -206,7 +252,11 @@ def main():
         "roofline": roof,
     }
     if not args.no_cpu_baseline:
-        out["cpu_baseline"] = cpu_baseline(A, B, N)
+        port = cpu_baseline(A, B, N)
+        ref = cpu_baseline_reference(A, B, N)
+        out["cpu_baseline"] = ref if ref is not None else port
+        if ref is not None:
+            out["cpu_baseline_all_cores"] = port
     print(json.dumps(out))
 
 

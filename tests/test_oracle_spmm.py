@@ -72,3 +72,38 @@ def test_compare_metric(oracle):
     rel, mx, mean = oracle.compare(c, ref)
     assert rel == pytest.approx(0.25)  # max(0.5/5, 0.25 absolute for the zero row)
     assert mx == pytest.approx(0.5) and mean == pytest.approx(0.75 / 4)
+
+
+def write_el(path, M, rp, ci, v):
+    """Edge list 'row col value' as CSR::read_from_edgelist (preprocess/src/general/csr.cpp:166-290) reads it."""
+    vals = v.view(np.float16).astype(np.float64)
+    with open(path, "w") as f:
+        for i in range(M):
+            for p in range(rp[i], rp[i + 1]):
+                f.write(f"{i} {ci[p]} {vals[p]:.10g}\n")
+
+
+@pytest.mark.parametrize("mb,density,N,seed", [(4, 0.5, 8, 11), (12, 0.2, 24, 12)])
+def test_against_reference_csr_multiply(oracle, tmp_path, mb, density, N, seed):
+    """The reference's own CSR::multiply (csr.cpp:47-63), compiled from the reference tree, on the same input."""
+    import subprocess
+    from tests.oracle_lib import ref_binary
+    exe = ref_binary("ref_csr_multiply")
+    if exe is None:
+        pytest.skip("oracle/_ref/ref_csr_multiply not built (reference tree absent)")
+    A = gen.random_bcsr(mb, mb, density, seed)  # square: the reference indexes B with A's row count
+    rp, ci, v = gen.bcsr_to_csr(A["M"], A["b_row_ptr"], A["b_col_idx"], A["b_val"])
+    # rows = last row + 1 and cols = largest column + 1 in the reference reader: pin both to M
+    assert rp[A["M"]] > rp[A["M"] - 1] and ci.max() <= A["M"] - 1
+    B = gen.dense_b(A["K"], N, seed + 1, dist="normal")
+    write_el(tmp_path / "a.el", A["M"], rp, ci, v)
+    B.view(np.float16).astype(np.float32).tofile(tmp_path / "b.f32")  # column-major, leading dimension K = M
+    out = subprocess.run([exe, str(tmp_path / "a.el"), str(tmp_path / "b.f32"), str(N), "1", str(tmp_path / "c.f32")],
+                         check=True, capture_output=True, text=True).stdout.split()
+    rows, cols, nnz = int(out[0]), int(out[1]), int(out[2])
+    assert rows == A["M"] and cols <= A["M"] and nnz == rp[A["M"]]
+    c_ref = np.fromfile(tmp_path / "c.f32", dtype=np.float32).reshape(N, rows).T  # column-major M x N
+    got = oracle.spmm_csr(A["M"], N, A["K"], rp, ci, v, B)
+    scale = np.abs(c_ref).max(axis=1, keepdims=True) + 1e-30
+    # same loop order; the two builds may differ in fused multiply-add contraction only
+    assert (np.abs(got - c_ref) / scale).max() < 1e-6
