@@ -33,6 +33,9 @@ MEASURED_TRAFFIC = {
 }
 
 
+INFO = {}  # facts about the generated workload that go into the config of the result line
+
+
 def build_workload(name):
     from smat_amd import generators as gen
     import smat_amd
@@ -49,9 +52,17 @@ def build_workload(name):
         b = smat_amd.csr_to_bcsr(d["M"], d["K"], d["row_ptr"], d["col_idx"], d["val"])
         A = {"M": b.M, "K": b.K, "b_row_ptr": b.row_ptr, "b_col_idx": b.col_idx, "b_val": b.val, "nnzb": b.nnzb}
         N, bdist, bseed = 64, "uniform", 0xB0000005
-    elif name == "er_16384_0.1pct_N256":
+    elif name in ("er_16384_0.1pct_N256", "er_16384_0.1pct_reordered_N256"):
         d = gen.erdos_renyi(16384, 0.001)
         b = smat_amd.csr_to_bcsr(d["M"], d["K"], d["row_ptr"], d["col_idx"], d["val"])
+        if "reordered" in name:
+            # row pass, then column pass on the transpose (-a 5 -b 16 -B 16 -F 1 -t 0.5), timed apart
+            t0 = time.perf_counter()
+            pr, pc, _, _ = smat_amd.reorder_csr(d["M"], d["K"], d["row_ptr"], d["col_idx"], 16, 16, 0.5, True)
+            INFO["reorder_s"] = round(time.perf_counter() - t0, 3)
+            INFO["nnzb_before_reorder"] = int(b.nnzb)
+            rp, ci, v = smat_amd.permute_csr(d["M"], d["K"], d["row_ptr"], d["col_idx"], d["val"], pr, pc)
+            b = smat_amd.csr_to_bcsr(d["M"], d["K"], rp, ci, v)
         A = {"M": b.M, "K": b.K, "b_row_ptr": b.row_ptr, "b_col_idx": b.col_idx, "b_val": b.val, "nnzb": b.nnzb}
         N, bdist, bseed = 256, "normal", 0xB0000002
     elif name == "rmat_s20_deg16_N128":
@@ -248,7 +259,7 @@ def main():
         "dtype": "f16",
         "data": "synthetic",
         "config": {"workload": args.workload, "M": M, "K": K, "N": N, "nnzb": nnzb, "block": 16,
-                   "c_dtype": "f16", "plan": None if plan is None else plan.info()},
+                   "c_dtype": "f16", "plan": None if plan is None else plan.info(), **INFO},
         "roofline": roof,
     }
     if not args.no_cpu_baseline:
