@@ -126,6 +126,14 @@ int smat_csr_to_bcsr(size_t M, size_t K, const int32_t *row_ptr, const int32_t *
                      int32_t **b_col_idx, uint16_t **b_val, int32_t **block_info,
                      int32_t **rel_map);
 
+/* The same conversion on the GPU: row_ptr / col_idx / val are DEVICE arrays (nnz = row_ptr[M]
+ * is passed by the caller), the three outputs are DEVICE arrays allocated by the library
+ * (release with smat_free) and hold exactly what smat_csr_to_bcsr returns for the same input,
+ * counts included.  row_ptr must be non-decreasing.  Synchronous. */
+int smat_csr_to_bcsr_device(size_t M, size_t K, const int32_t *row_ptr, const int32_t *col_idx,
+                            const uint16_t *val, size_t nnz, int64_t *counts, int32_t **b_row_ptr,
+                            int32_t **b_col_idx, uint16_t **b_val);
+
 /* ---- reorder (host) --------------------------------------------------------
  * Row clustering that minimises the number of nonzero blocks: the reference's
  * `Matrix_Blocking -a 5 -F 1` path, BlockingEngine::GetGrouping

@@ -10,6 +10,8 @@ from .host import (  # noqa: F401
     Bcsr,
     Plan,
     csr_to_bcsr,
+    csr_to_bcsr_device,
+    DeviceBcsr,
     mtx_read,
     permute_csr,
     reorder_csr,
@@ -18,6 +20,6 @@ from .host import (  # noqa: F401
 )
 
 __all__ = [
-    "lib", "SmatError", "library_path", "Bcsr", "Plan", "csr_to_bcsr", "mtx_read",
+    "lib", "SmatError", "library_path", "Bcsr", "Plan", "csr_to_bcsr", "csr_to_bcsr_device", "DeviceBcsr", "mtx_read",
     "permute_csr", "reorder_csr", "reorder_rows", "spmm",
 ]

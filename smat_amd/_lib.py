@@ -43,6 +43,7 @@ SIGNATURES = {
                               _pp, _pp, _pp, C.POINTER(_int)]),
     "smat_host_free": (None, [_vp]),
     "smat_csr_to_bcsr": (_int, [_sz, _sz, _vp, _vp, _vp, _pi64, _pp, _pp, _pp, _pp, _pp]),
+    "smat_csr_to_bcsr_device": (_int, [_sz, _sz, _vp, _vp, _vp, _sz, _pi64, _pp, _pp, _pp]),
     "smat_reorder_rows": (_int, [_i64, _i64, _vp, _vp, _i64, _i64, C.c_float, _vp, _vp, _vp]),
     "smat_reorder_csr": (_int, [_sz, _sz, _vp, _vp, _i64, _i64, C.c_float, _int, _vp, _vp, _vp, _vp]),
     "smat_permute_csr": (_int, [_sz, _sz, _vp, _vp, _vp, _vp, _vp, _pp, _pp, _pp]),

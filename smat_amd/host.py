@@ -79,6 +79,50 @@ def csr_to_bcsr(M, K, row_ptr, col_idx, val, want_maps=False):
     return out
 
 
+class DeviceBcsr:
+    """BCSR arrays in device memory, as returned by smat_csr_to_bcsr_device (freed on close)."""
+
+    def __init__(self, M, K, row_ptr, col_idx, val, counts):
+        self.M, self.K, self.counts = M, K, counts
+        self.row_ptr, self.col_idx, self.val = row_ptr, col_idx, val  # device addresses (ints)
+
+    @property
+    def nnzb(self):
+        return int(self.counts[0])
+
+    def to_host(self):
+        rp = np.empty(self.M // BS + 1, np.int32)
+        ci = np.empty(self.nnzb, np.int32)
+        v = np.empty(self.nnzb * 256, np.uint16)
+        check(lib.smat_memcpy_d2h(_p(rp), self.row_ptr, rp.nbytes))
+        if self.nnzb:
+            check(lib.smat_memcpy_d2h(_p(ci), self.col_idx, ci.nbytes))
+            check(lib.smat_memcpy_d2h(_p(v), self.val, v.nbytes))
+        return Bcsr(self.M, self.K, rp, ci, v, tuple(self.counts))
+
+    def close(self):
+        for a in ("row_ptr", "col_idx", "val"):
+            if getattr(self, a):
+                lib.smat_free(getattr(self, a))
+                setattr(self, a, None)
+
+    def __del__(self):
+        try:
+            self.close()
+        except Exception:
+            pass
+
+
+def csr_to_bcsr_device(M, K, row_ptr_dev, col_idx_dev, val_dev, nnz):
+    """CSR -> BCSR on the GPU; the three inputs are device tensors (anything with .data_ptr())."""
+    counts = (C.c_int64 * 3)()
+    brp, bci, bv = C.c_void_p(), C.c_void_p(), C.c_void_p()
+    ptr = lambda t: C.c_void_p(t.data_ptr()) if t is not None else None  # noqa: E731
+    check(lib.smat_csr_to_bcsr_device(M, K, ptr(row_ptr_dev), ptr(col_idx_dev), ptr(val_dev), nnz, counts,
+                                      C.byref(brp), C.byref(bci), C.byref(bv)))
+    return DeviceBcsr(M, K, brp.value, bci.value, bv.value, tuple(counts))
+
+
 def reorder_rows(rows, cols, row_ptr, col_idx, col_block=16, row_block=16, tau=0.5):
     """One pass of the row clustering. Returns (grouping, perm, stats)."""
     row_ptr = np.ascontiguousarray(row_ptr, dtype=np.int64)
