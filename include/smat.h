@@ -114,6 +114,30 @@ int smat_mtx_read(const char *path, size_t *M, size_t *K, size_t *nnz, int *is_s
                   int32_t **row_ptr, int32_t **col_idx, uint16_t **val, int *ref_code);
 void smat_host_free(void *p);
 
+/* ---- binary container (host) ----------------------------------------------
+ * The reference keeps matrices as text only (.mtx read by mmio_allinone,
+ * mmio_highlevel.h:619-786; .el for the reorder program, csr.cpp:153-290).  A
+ * "SMATBIN1" file holds the same arrays in binary, optionally with the row and
+ * column permutations of a reorder, behind a 64-byte header with a checksum.
+ * kind: 1 = CSR (n = nnz, val = n halfs), 2 = BCSR (n = nonzero blocks,
+ * row_ptr has M/16+1 entries, val = n*256 halfs).  perm_* may be NULL on write;
+ * on read, pass NULL to skip them, and expect NULL back when the file has none.
+ * Arrays returned by smat_bin_read are released with smat_host_free. */
+#define SMAT_BIN_CSR 1
+#define SMAT_BIN_BCSR 2
+int smat_bin_write_csr(const char *path, size_t M, size_t K, const int32_t *row_ptr,
+                       const int32_t *col_idx, const uint16_t *val, const int64_t *perm_rows,
+                       const int64_t *perm_cols);
+int smat_bin_write_bcsr(const char *path, size_t M, size_t K, size_t nnzb, const int32_t *b_row_ptr,
+                        const int32_t *b_col_idx, const uint16_t *b_val, const int64_t *perm_rows,
+                        const int64_t *perm_cols);
+int smat_bin_read(const char *path, int *kind, size_t *M, size_t *K, size_t *n, int32_t **row_ptr,
+                  int32_t **col_idx, uint16_t **val, int64_t **perm_rows, int64_t **perm_cols);
+/* CSR -> Matrix Market "coordinate real general" (entries in storage order): the way back
+ * to the reference's text format; smat_mtx_read of the result returns the same CSR. */
+int smat_mtx_write(const char *path, size_t M, size_t K, const int32_t *row_ptr,
+                   const int32_t *col_idx, const uint16_t *val);
+
 /* ---- blocking: CSR -> 16x16 BCSR (host) -----------------------------------
  * Replaces SparseMatrix::csrToBcsr (src/cuda_hgemm/src/common/matrix.h:376-502)
  * and emits bit-identical row_ptr / col_idx / val without the two dense

@@ -10,6 +10,10 @@ from .host import (  # noqa: F401
     Bcsr,
     Plan,
     csr_to_bcsr,
+    bin_write_csr,
+    bin_write_bcsr,
+    bin_read,
+    mtx_write,
     csr_to_bcsr_device,
     DeviceBcsr,
     mtx_read,
@@ -20,6 +24,6 @@ from .host import (  # noqa: F401
 )
 
 __all__ = [
-    "lib", "SmatError", "library_path", "Bcsr", "Plan", "csr_to_bcsr", "csr_to_bcsr_device", "DeviceBcsr", "mtx_read",
+    "lib", "SmatError", "library_path", "Bcsr", "Plan", "csr_to_bcsr", "bin_write_csr", "bin_write_bcsr", "bin_read", "mtx_write", "csr_to_bcsr_device", "DeviceBcsr", "mtx_read",
     "permute_csr", "reorder_csr", "reorder_rows", "spmm",
 ]

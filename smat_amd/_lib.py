@@ -42,6 +42,11 @@ SIGNATURES = {
     "smat_mtx_read": (_int, [C.c_char_p, C.POINTER(_sz), C.POINTER(_sz), C.POINTER(_sz), C.POINTER(_int),
                               _pp, _pp, _pp, C.POINTER(_int)]),
     "smat_host_free": (None, [_vp]),
+    "smat_bin_write_csr": (_int, [C.c_char_p, _sz, _sz, _vp, _vp, _vp, _vp, _vp]),
+    "smat_bin_write_bcsr": (_int, [C.c_char_p, _sz, _sz, _sz, _vp, _vp, _vp, _vp, _vp]),
+    "smat_bin_read": (_int, [C.c_char_p, C.POINTER(_int), C.POINTER(_sz), C.POINTER(_sz), C.POINTER(_sz),
+                              _pp, _pp, _pp, _pp, _pp]),
+    "smat_mtx_write": (_int, [C.c_char_p, _sz, _sz, _vp, _vp, _vp]),
     "smat_csr_to_bcsr": (_int, [_sz, _sz, _vp, _vp, _vp, _pi64, _pp, _pp, _pp, _pp, _pp]),
     "smat_csr_to_bcsr_device": (_int, [_sz, _sz, _vp, _vp, _vp, _sz, _pi64, _pp, _pp, _pp]),
     "smat_reorder_rows": (_int, [_i64, _i64, _vp, _vp, _i64, _i64, C.c_float, _vp, _vp, _vp]),

@@ -59,8 +59,18 @@ class SparseMatrix {
 public:
     SparseMatrix(const std::string &name, const std::string &file, bool reorder, float tau) : name_(name)
     {
-        int sym = 0;
-        SMAT_CHECK(smat_mtx_read(file.c_str(), &row_, &col_, &nnz_, &sym, &csrRowPtr_, &csrColIdx_, &csrVal_, nullptr));
+        if (isContainer(file)) {  // binary CSR container written by smat_convert: no text parse
+            int kind = 0;
+            SMAT_CHECK(smat_bin_read(file.c_str(), &kind, &row_, &col_, &nnz_, &csrRowPtr_, &csrColIdx_, &csrVal_,
+                                     nullptr, nullptr));
+            if (kind != SMAT_BIN_CSR || row_ % 16 || col_ % 16) {
+                HLOG("%s: expected a CSR container with dimensions padded to multiples of 16", file.c_str());
+                exit(EXIT_FAILURE);
+            }
+        } else {
+            int sym = 0;
+            SMAT_CHECK(smat_mtx_read(file.c_str(), &row_, &col_, &nnz_, &sym, &csrRowPtr_, &csrColIdx_, &csrVal_, nullptr));
+        }
         HLOG("Read %s", file.c_str());
         if (!row_ || !col_ || !nnz_) { HLOG("empty matrix"); exit(EXIT_FAILURE); }
         HLOG("%zu x %zu, nnz = %zu, A[0] = %f", row_, col_, nnz_, smat::half_to_float(csrVal_[0]));
@@ -92,6 +102,15 @@ public:
         SMAT_CHECK(smat_memcpy_h2d(bcsrVal_dev_, bcsrVal_, nonzeroBlocks_ * 256 * sizeof(half)));
         SMAT_CHECK(smat_memcpy_h2d(bcsrColIdx_dev_, bcsrColIdx_, nonzeroBlocks_ * sizeof(int)));
         SMAT_CHECK(smat_memcpy_h2d(bcsrRowPtr_dev_, bcsrRowPtr_, (row_ / 16 + 1) * sizeof(int)));
+    }
+    static bool isContainer(const std::string &file)
+    {
+        FILE *f = fopen(file.c_str(), "rb");
+        if (!f) return false;
+        char m[8] = {0};
+        const bool ok = fread(m, 1, 8, f) == 8 && memcmp(m, "SMATBIN1", 8) == 0;
+        fclose(f);
+        return ok;
     }
     ~SparseMatrix()
     {

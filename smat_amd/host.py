@@ -43,6 +43,52 @@ def mtx_read(path):
     }
 
 
+def bin_write_csr(path, M, K, row_ptr, col_idx, val, perm_rows=None, perm_cols=None):
+    """CSR (+ optional permutations) -> SMATBIN1 container."""
+    row_ptr = np.ascontiguousarray(row_ptr, dtype=np.int32)
+    col_idx = np.ascontiguousarray(col_idx, dtype=np.int32)
+    val = np.ascontiguousarray(val, dtype=np.uint16)
+    pr = None if perm_rows is None else np.ascontiguousarray(perm_rows, dtype=np.int64)
+    pc = None if perm_cols is None else np.ascontiguousarray(perm_cols, dtype=np.int64)
+    check(lib.smat_bin_write_csr(str(path).encode(), M, K, _p(row_ptr), _p(col_idx), _p(val), _p(pr), _p(pc)))
+
+
+def bin_write_bcsr(path, M, K, b_row_ptr, b_col_idx, b_val, perm_rows=None, perm_cols=None):
+    """16x16 BCSR (+ optional permutations) -> SMATBIN1 container."""
+    b_row_ptr = np.ascontiguousarray(b_row_ptr, dtype=np.int32)
+    b_col_idx = np.ascontiguousarray(b_col_idx, dtype=np.int32)
+    b_val = np.ascontiguousarray(b_val, dtype=np.uint16)
+    pr = None if perm_rows is None else np.ascontiguousarray(perm_rows, dtype=np.int64)
+    pc = None if perm_cols is None else np.ascontiguousarray(perm_cols, dtype=np.int64)
+    check(lib.smat_bin_write_bcsr(str(path).encode(), M, K, len(b_col_idx), _p(b_row_ptr), _p(b_col_idx), _p(b_val),
+                                  _p(pr), _p(pc)))
+
+
+def bin_read(path):
+    """SMATBIN1 container -> dict(kind, M, K, n, row_ptr, col_idx, val, perm_rows, perm_cols)."""
+    kind, M, K, n = C.c_int(), C.c_size_t(), C.c_size_t(), C.c_size_t()
+    rp, ci, v, pr, pc = C.c_void_p(), C.c_void_p(), C.c_void_p(), C.c_void_p(), C.c_void_p()
+    check(lib.smat_bin_read(str(path).encode(), C.byref(kind), C.byref(M), C.byref(K), C.byref(n), C.byref(rp),
+                            C.byref(ci), C.byref(v), C.byref(pr), C.byref(pc)))
+    rows = M.value if kind.value == 1 else M.value // BS
+    per = 1 if kind.value == 1 else 256
+    return {
+        "kind": kind.value, "M": M.value, "K": K.value, "n": n.value,
+        "row_ptr": _take(rp, rows + 1, np.int32), "col_idx": _take(ci, n.value, np.int32),
+        "val": _take(v, n.value * per, np.uint16),
+        "perm_rows": _take(pr, M.value, np.int64) if pr.value else None,
+        "perm_cols": _take(pc, K.value, np.int64) if pc.value else None,
+    }
+
+
+def mtx_write(path, M, K, row_ptr, col_idx, val):
+    """CSR -> Matrix Market coordinate real general, entries in storage order."""
+    row_ptr = np.ascontiguousarray(row_ptr, dtype=np.int32)
+    col_idx = np.ascontiguousarray(col_idx, dtype=np.int32)
+    val = np.ascontiguousarray(val, dtype=np.uint16)
+    check(lib.smat_mtx_write(str(path).encode(), M, K, _p(row_ptr), _p(col_idx), _p(val)))
+
+
 @dataclass
 class Bcsr:
     M: int

@@ -1,0 +1,109 @@
+"""Binary container: exact round trips, rejection of damaged files, text <-> binary conversion."""
+import os
+import subprocess
+
+import numpy as np
+import pytest
+
+import smat_amd
+from smat_amd import generators as gen
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+BIN = os.path.join(ROOT, "smat_amd", "bin")
+
+
+def all_halfs_csr():
+    """A 4096-row matrix whose values run over every finite fp16 bit pattern once."""
+    bits = np.array([b for b in range(0x10000) if (b & 0x7C00) != 0x7C00], dtype=np.uint16)
+    M = K = 4096
+    rows = np.arange(bits.size) % M
+    order = np.argsort(rows, kind="stable")
+    rp = np.zeros(M + 1, np.int32)
+    np.add.at(rp, rows + 1, 1)
+    rp = np.cumsum(rp).astype(np.int32)
+    ci = ((np.arange(bits.size) * 37) % K).astype(np.int32)[order]
+    return M, K, rp, ci, bits[order]
+
+
+def test_csr_round_trip_with_permutations(tmp_path):
+    d = gen.erdos_renyi(512, 0.01, seed=3)
+    rng = np.random.default_rng(1)
+    pr, pc = rng.permutation(d["M"]).astype(np.int64), rng.permutation(d["K"]).astype(np.int64)
+    path = tmp_path / "a.smat"
+    smat_amd.bin_write_csr(path, d["M"], d["K"], d["row_ptr"], d["col_idx"], d["val"], pr, pc)
+    assert os.path.getsize(path) % 64 == 0
+    r = smat_amd.bin_read(path)
+    assert (r["kind"], r["M"], r["K"], r["n"]) == (1, d["M"], d["K"], int(d["row_ptr"][-1]))
+    for k in ("row_ptr", "col_idx", "val"):
+        assert np.array_equal(r[k], d[k])
+    assert np.array_equal(r["perm_rows"], pr) and np.array_equal(r["perm_cols"], pc)
+    # without permutations: NULL comes back
+    smat_amd.bin_write_csr(path, d["M"], d["K"], d["row_ptr"], d["col_idx"], d["val"])
+    r = smat_amd.bin_read(path)
+    assert r["perm_rows"] is None and r["perm_cols"] is None
+
+
+def test_bcsr_round_trip_and_empty(tmp_path):
+    A = gen.random_bcsr(9, 13, 0.3, seed=4)
+    path = tmp_path / "b.smat"
+    smat_amd.bin_write_bcsr(path, A["M"], A["K"], A["b_row_ptr"], A["b_col_idx"], A["b_val"])
+    r = smat_amd.bin_read(path)
+    assert r["kind"] == 2 and r["n"] == len(A["b_col_idx"])
+    assert np.array_equal(r["row_ptr"], A["b_row_ptr"]) and np.array_equal(r["col_idx"], A["b_col_idx"])
+    assert np.array_equal(r["val"], A["b_val"])
+    smat_amd.bin_write_bcsr(path, 32, 48, np.zeros(3, np.int32), np.zeros(0, np.int32), np.zeros(0, np.uint16))
+    r = smat_amd.bin_read(path)
+    assert r["n"] == 0 and r["row_ptr"].tolist() == [0, 0, 0]
+
+
+def test_damaged_files_are_rejected(tmp_path):
+    d = gen.band(256, 8)
+    path = tmp_path / "a.smat"
+    smat_amd.bin_write_csr(path, d["M"], d["K"], d["row_ptr"], d["col_idx"], d["val"])
+    raw = bytearray(path.read_bytes())
+    (tmp_path / "trunc.smat").write_bytes(raw[: len(raw) // 2])
+    flipped = bytearray(raw); flipped[200] ^= 0x40
+    (tmp_path / "flip.smat").write_bytes(flipped)
+    magic = bytearray(raw); magic[0:4] = b"XXXX"
+    (tmp_path / "magic.smat").write_bytes(magic)
+    for name, text in (("trunc.smat", "truncated"), ("flip.smat", "checksum"), ("magic.smat", "not a SMATBIN1"),
+                       ("missing.smat", "cannot open")):
+        with pytest.raises(smat_amd.SmatError, match=text):
+            smat_amd.bin_read(tmp_path / name)
+
+
+def test_text_round_trip_keeps_every_half(tmp_path):
+    M, K, rp, ci, v = all_halfs_csr()
+    smat_amd.mtx_write(tmp_path / "all.mtx", M, K, rp, ci, v)
+    r = smat_amd.mtx_read(tmp_path / "all.mtx")
+    assert (r["M"], r["K"]) == (M, K)
+    assert np.array_equal(r["row_ptr"], rp) and np.array_equal(r["col_idx"], ci)
+    assert np.array_equal(r["val"], v)  # -0.0 and subnormals included
+
+
+def test_converter_cli(tmp_path):
+    d = gen.erdos_renyi(256, 0.02, seed=9)
+    smat_amd.mtx_write(tmp_path / "a.mtx", d["M"], d["K"], d["row_ptr"], d["col_idx"], d["val"])
+    conv = os.path.join(BIN, "smat_convert")
+    subprocess.run([conv, "-in", str(tmp_path / "a.mtx"), "-out", str(tmp_path / "a.smat")], check=True,
+                   stdout=subprocess.DEVNULL)
+    r = smat_amd.bin_read(tmp_path / "a.smat")
+    want = smat_amd.mtx_read(tmp_path / "a.mtx")
+    for k in ("row_ptr", "col_idx", "val"):
+        assert np.array_equal(r[k], want[k])
+    # back to text: same CSR again
+    subprocess.run([conv, "-in", str(tmp_path / "a.smat"), "-out", str(tmp_path / "b.mtx")], check=True,
+                   stdout=subprocess.DEVNULL)
+    again = smat_amd.mtx_read(tmp_path / "b.mtx")
+    for k in ("row_ptr", "col_idx", "val"):
+        assert np.array_equal(again[k], want[k])
+    # reorder + block ahead of time: the container holds what the in-process calls produce
+    subprocess.run([conv, "-in", str(tmp_path / "a.mtx"), "-out", str(tmp_path / "c.smat"), "-reorder", "-bcsr"],
+                   check=True, stdout=subprocess.DEVNULL)
+    c = smat_amd.bin_read(tmp_path / "c.smat")
+    pr, pc, _, _ = smat_amd.reorder_csr(want["M"], want["K"], want["row_ptr"], want["col_idx"], 16, 16, 0.5, True)
+    rp, ci, v = smat_amd.permute_csr(want["M"], want["K"], want["row_ptr"], want["col_idx"], want["val"], pr, pc)
+    b = smat_amd.csr_to_bcsr(want["M"], want["K"], rp, ci, v)
+    assert c["kind"] == 2 and np.array_equal(c["perm_rows"], pr) and np.array_equal(c["perm_cols"], pc)
+    assert np.array_equal(c["row_ptr"], b.row_ptr) and np.array_equal(c["col_idx"], b.col_idx)
+    assert np.array_equal(c["val"], b.val)

@@ -71,3 +71,18 @@ def test_hgemm_flow_with_check(tmp_path, extra):
     assert run.returncode == 0, run.stderr[-2000:]
     assert "PASS" in run.stderr and "1008 x 1008" in run.stderr and "Done" in run.stderr
     assert (tmp_path / "results_smat.csv").read_text().startswith(str(mtx) + ",")
+
+
+@pytest.mark.gpu
+def test_hgemm_reads_binary_container(tmp_path):
+    """The text parse can be done once, ahead of time: hgemm takes the SMATBIN1 file smat_convert writes."""
+    d = gen.stencil27(10)
+    mtx = tmp_path / "stencil10.mtx"
+    write_mtx(mtx, d)
+    subprocess.run([os.path.join(BIN, "smat_convert"), "-in", str(mtx), "-out", str(tmp_path / "stencil10.smat")],
+                   check=True, stdout=subprocess.DEVNULL)
+    cmd = [os.path.join(BIN, "hgemm"), f"-filename={tmp_path / 'stencil10.smat'}", "-n_mult=9", "-enable_check",
+           "-random_b", "-warmup_iterations=1", "-profiling_iterations=3", "-sleep_duration=1", "-use_plan"]
+    run = subprocess.run(cmd, cwd=tmp_path, capture_output=True, text=True, timeout=120)
+    assert run.returncode == 0, run.stderr[-2000:]
+    assert "PASS" in run.stderr and "1008 x 1008" in run.stderr
