@@ -29,7 +29,9 @@ PEAK_HBM_GBS = 8000.0      # MI355X HBM3E
 # HBM bytes per launch measured with rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE and scaled by a plain
 # device copy of known size (summaries under profiles/): (workload, kernel id) -> bytes
 MEASURED_TRAFFIC = {
-    ("block_pruned_8192_10pct_N4096", 2): 143441 * 1024 * 2.0 + 65851 * 1024 * 1.0,
+    ("block_pruned_8192_10pct_N4096", 2): 143442 * 1024 * 2.0 + 65824 * 1024 * 1.0,
+    # row-wise kernel + repack kernel
+    ("er_16384_0.1pct_reordered_N256", 1): (225508 + 4110) * 1024 * 2.0 + (8192 + 8192) * 1024 * 1.0,
 }
 
 
