@@ -4,7 +4,9 @@
 //   -enable_check -gpu_rank -cpu_procs  (-M -N -K -enable_wmma -enable_mma are
 //   accepted and ignored: they only sized the dense-GEMM leftovers there)
 // and adds: -reorder (row + column clustering before blocking), -tau,
-//   -random_b (seeded uniform[-1,1] B instead of all ones), -use_plan, -kernel.
+//   -random_b (seeded uniform[-1,1] B instead of all ones), -use_plan, -kernel,
+//   -gpu_blocking (CSR -> BCSR on the device).  -filename also takes a binary container
+//   written by smat_convert.  Load, reorder and blocking times are logged apart from the SpMM time.
 #include <thread>
 
 #include "flags.h"
@@ -35,7 +37,7 @@ int main(int argc, char **argv)
     Tester tester((size_t)f.num("warmup_iterations", 1), (size_t)f.num("profiling_iterations", 10),
                   (size_t)f.num("sleep_duration", 100), f.flag("enable_check", false), n_mult, file,
                   f.flag("reorder", false), (float)f.real("tau", 0.5), f.flag("random_b", false),
-                  f.flag("use_plan", true), (int)f.num("kernel", SMAT_KERNEL_AUTO));
+                  f.flag("use_plan", true), (int)f.num("kernel", SMAT_KERNEL_AUTO), f.flag("gpu_blocking", false));
     if (f.flag("use_plan", true))
         tester.evaluatePlanned("Smat-Plan-Kernel");
     else

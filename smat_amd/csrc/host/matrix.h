@@ -4,7 +4,9 @@
 // device memory goes through the C ABI, there is no HIP header here.
 #pragma once
 #include <cmath>
+#include <cstdlib>
 #include <cstring>
+#include <ctime>
 #include <random>
 #include <string>
 #include <vector>
@@ -57,8 +59,12 @@ private:
 
 class SparseMatrix {
 public:
-    SparseMatrix(const std::string &name, const std::string &file, bool reorder, float tau) : name_(name)
+    // gpu_blocking: CSR -> BCSR on the device (smat_csr_to_bcsr_device) instead of on the host;
+    // the arrays are the same, the host copies are fetched back for the plan and the verify step.
+    SparseMatrix(const std::string &name, const std::string &file, bool reorder, float tau, bool gpu_blocking = false)
+        : name_(name)
     {
+        double t0 = wallMs();
         if (isContainer(file)) {  // binary CSR container written by smat_convert: no text parse
             int kind = 0;
             SMAT_CHECK(smat_bin_read(file.c_str(), &kind, &row_, &col_, &nnz_, &csrRowPtr_, &csrColIdx_, &csrVal_,
@@ -71,9 +77,10 @@ public:
             int sym = 0;
             SMAT_CHECK(smat_mtx_read(file.c_str(), &row_, &col_, &nnz_, &sym, &csrRowPtr_, &csrColIdx_, &csrVal_, nullptr));
         }
-        HLOG("Read %s", file.c_str());
+        HLOG("Read %s in %.1f ms", file.c_str(), wallMs() - t0);
         if (!row_ || !col_ || !nnz_) { HLOG("empty matrix"); exit(EXIT_FAILURE); }
         HLOG("%zu x %zu, nnz = %zu, A[0] = %f", row_, col_, nnz_, smat::half_to_float(csrVal_[0]));
+        t0 = wallMs();
         if (reorder) {  // row pass + column pass, values kept (the reference pipeline drops them: src/reorder.py:38-40)
             permRows_.resize(row_);
             permCols_.resize(col_);
@@ -88,20 +95,53 @@ public:
             csrRowPtr_ = rp; csrColIdx_ = ci; csrVal_ = v;
             HLOG("Reordered: row pass %lld nonzero blocks (%lld comparisons), column pass %lld (%lld comparisons)",
                  (long long)sr[2], (long long)sr[0], (long long)sc[2], (long long)sc[0]);
+            HLOG("Reorder time: %.1f ms (host, not part of the SpMM time)", wallMs() - t0);
         }
         int64_t counts[3];
-        SMAT_CHECK(smat_csr_to_bcsr(row_, col_, csrRowPtr_, csrColIdx_, csrVal_, counts, &bcsrRowPtr_, &bcsrColIdx_,
-                                    &bcsrVal_, nullptr, nullptr));
-        nonzeroBlocks_ = (size_t)counts[0];
+        t0 = wallMs();
+        if (gpu_blocking) {
+            int32_t *rp_d, *ci_d;
+            uint16_t *v_d;
+            SMAT_CHECK(smat_malloc((void **)&rp_d, (row_ + 1) * sizeof(int)));
+            SMAT_CHECK(smat_malloc((void **)&ci_d, nnz_ * sizeof(int)));
+            SMAT_CHECK(smat_malloc((void **)&v_d, nnz_ * sizeof(half)));
+            SMAT_CHECK(smat_memcpy_h2d(rp_d, csrRowPtr_, (row_ + 1) * sizeof(int)));
+            SMAT_CHECK(smat_memcpy_h2d(ci_d, csrColIdx_, nnz_ * sizeof(int)));
+            SMAT_CHECK(smat_memcpy_h2d(v_d, csrVal_, nnz_ * sizeof(half)));
+            const double t1 = wallMs();
+            SMAT_CHECK(smat_csr_to_bcsr_device(row_, col_, rp_d, ci_d, v_d, nnz_, counts, &bcsrRowPtr_dev_,
+                                               &bcsrColIdx_dev_, (uint16_t **)&bcsrVal_dev_));
+            HLOG("Blocking on the GPU: %.1f ms (+ %.1f ms to copy the CSR to the device)", wallMs() - t1, t1 - t0);
+            smat_free(rp_d); smat_free(ci_d); smat_free(v_d);
+            nonzeroBlocks_ = (size_t)counts[0];
+            bcsrRowPtr_ = (int32_t *)malloc((row_ / 16 + 1) * sizeof(int));
+            bcsrColIdx_ = (int32_t *)malloc(std::max<size_t>(nonzeroBlocks_, 1) * sizeof(int));
+            bcsrVal_ = (uint16_t *)malloc(std::max<size_t>(nonzeroBlocks_, 1) * 256 * sizeof(half));
+            if (!bcsrRowPtr_ || !bcsrColIdx_ || !bcsrVal_) { HLOG("out of host memory"); exit(EXIT_FAILURE); }
+            SMAT_CHECK(smat_memcpy_d2h(bcsrRowPtr_, bcsrRowPtr_dev_, (row_ / 16 + 1) * sizeof(int)));
+            SMAT_CHECK(smat_memcpy_d2h(bcsrColIdx_, bcsrColIdx_dev_, nonzeroBlocks_ * sizeof(int)));
+            SMAT_CHECK(smat_memcpy_d2h(bcsrVal_, bcsrVal_dev_, nonzeroBlocks_ * 256 * sizeof(half)));
+        } else {
+            SMAT_CHECK(smat_csr_to_bcsr(row_, col_, csrRowPtr_, csrColIdx_, csrVal_, counts, &bcsrRowPtr_, &bcsrColIdx_,
+                                        &bcsrVal_, nullptr, nullptr));
+            nonzeroBlocks_ = (size_t)counts[0];
+            HLOG("Blocking on the host: %.1f ms", wallMs() - t0);
+            SMAT_CHECK(smat_malloc((void **)&bcsrVal_dev_, nonzeroBlocks_ * 256 * sizeof(half)));
+            SMAT_CHECK(smat_malloc((void **)&bcsrColIdx_dev_, nonzeroBlocks_ * sizeof(int)));
+            SMAT_CHECK(smat_malloc((void **)&bcsrRowPtr_dev_, (row_ / 16 + 1) * sizeof(int)));
+            SMAT_CHECK(smat_memcpy_h2d(bcsrVal_dev_, bcsrVal_, nonzeroBlocks_ * 256 * sizeof(half)));
+            SMAT_CHECK(smat_memcpy_h2d(bcsrColIdx_dev_, bcsrColIdx_, nonzeroBlocks_ * sizeof(int)));
+            SMAT_CHECK(smat_memcpy_h2d(bcsrRowPtr_dev_, bcsrRowPtr_, (row_ / 16 + 1) * sizeof(int)));
+        }
         HLOG("Finished creating BCSR from CSR");
         HLOG("%zu total blocks, %zu nonzero blocks, %zu dense blocks, %zu sparse blocks", (row_ / 16) * (col_ / 16),
              nonzeroBlocks_, (size_t)counts[1], (size_t)counts[2]);
-        SMAT_CHECK(smat_malloc((void **)&bcsrVal_dev_, nonzeroBlocks_ * 256 * sizeof(half)));
-        SMAT_CHECK(smat_malloc((void **)&bcsrColIdx_dev_, nonzeroBlocks_ * sizeof(int)));
-        SMAT_CHECK(smat_malloc((void **)&bcsrRowPtr_dev_, (row_ / 16 + 1) * sizeof(int)));
-        SMAT_CHECK(smat_memcpy_h2d(bcsrVal_dev_, bcsrVal_, nonzeroBlocks_ * 256 * sizeof(half)));
-        SMAT_CHECK(smat_memcpy_h2d(bcsrColIdx_dev_, bcsrColIdx_, nonzeroBlocks_ * sizeof(int)));
-        SMAT_CHECK(smat_memcpy_h2d(bcsrRowPtr_dev_, bcsrRowPtr_, (row_ / 16 + 1) * sizeof(int)));
+    }
+    static double wallMs()
+    {
+        struct timespec ts;
+        clock_gettime(CLOCK_MONOTONIC, &ts);
+        return ts.tv_sec * 1e3 + ts.tv_nsec * 1e-6;
     }
     static bool isContainer(const std::string &file)
     {

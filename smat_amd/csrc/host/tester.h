@@ -26,12 +26,13 @@
 class Tester {
 public:
     Tester(size_t warmup_iterations, size_t profiling_iterations, size_t sleep_duration, bool enable_check,
-           int n_mult, const std::string &filename, bool reorder, float tau, bool random_b, bool use_plan, int kernel)
+           int n_mult, const std::string &filename, bool reorder, float tau, bool random_b, bool use_plan, int kernel,
+           bool gpu_blocking = false)
         : warmup_(warmup_iterations), iters_(profiling_iterations), sleep_ms_(sleep_duration), check_(enable_check),
           file_(filename), kernel_(kernel)
     {
         if (!warmup_ || !iters_) { HLOG("warmup_iterations and profiling_iterations must be positive"); exit(EXIT_FAILURE); }
-        A_ = new SparseMatrix("Sparse Matrix A", filename, reorder, tau);
+        A_ = new SparseMatrix("Sparse Matrix A", filename, reorder, tau, gpu_blocking);
         const size_t N = (size_t)n_mult * 8; // MMA_N of the reference, tester.h:40
         B_ = new Matrix(A_->getCol(), N, "Matrix B for sparse", random_b, 0xB);
         C_ = new Matrix(A_->getRow(), N, "Matrix C for sparse");

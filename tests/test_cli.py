@@ -86,3 +86,10 @@ def test_hgemm_reads_binary_container(tmp_path):
     run = subprocess.run(cmd, cwd=tmp_path, capture_output=True, text=True, timeout=120)
     assert run.returncode == 0, run.stderr[-2000:]
     assert "PASS" in run.stderr and "1008 x 1008" in run.stderr
+    # same flow with the blocking done on the GPU: same block counts in the log, same verdict
+    run2 = subprocess.run(cmd + ["-gpu_blocking"], cwd=tmp_path, capture_output=True, text=True, timeout=120)
+    assert run2.returncode == 0, run2.stderr[-2000:]
+    assert "PASS" in run2.stderr and "Blocking on the GPU" in run2.stderr
+    blocks = [ln.split("]")[-1] for ln in run.stderr.splitlines() if "nonzero blocks," in ln]
+    blocks2 = [ln.split("]")[-1] for ln in run2.stderr.splitlines() if "nonzero blocks," in ln]
+    assert blocks and blocks == blocks2
