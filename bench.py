@@ -5,7 +5,8 @@ A "step" is one SpMM launch C = A_bcsr x B over inputs already resident in HBM.
 Default workload = the block-pruned configuration the metric is quoted on:
 A 8192 x 8192 fp16, 16x16 block mask with 10% of the blocks kept (dense inside,
 N(0, 0.02)), B 8192 x 4096 fp16 N(0,1), fp16 C.  The work list (plan) is built
-once, outside the timed region, like the reference builds its BCSR once.
+once, outside the timed region, like the reference builds its BCSR once; it also
+looks at the block values once (which columns of the blocks are nonzero).
 
 Prints ONE JSON line: effective GFLOP/s = 2 * nnzb * 256 * N / t, the roofline
 fraction of the SpMM kernel (timed with HIP events on the launch stream), and a
@@ -163,9 +164,11 @@ def main():
     ap.add_argument("--steps", type=int, default=200)
     ap.add_argument("--warmup", type=int, default=20)
     ap.add_argument("--workload", default="block_pruned_8192_10pct_N4096")
-    ap.add_argument("--kernel", type=int, default=0, help="0 auto, 1 rowwise, 2 sweep, 3 rowwise reading B in place")
+    ap.add_argument("--kernel", type=int, default=0, help="0 auto, 1 rowwise, 2 sweep, 3 rowwise reading B in place, 5 compact")
     ap.add_argument("--no-plan", action="store_true")
     ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--no-attach-values", action="store_true",
+                    help="do not let the plan look at the block values (the compact kernel, id 5, needs them)")
     ap.add_argument("--calibration-copy-mib", type=int, default=0,
                     help="also run one plain device copy of this many MiB (a kernel of known HBM traffic, "
                          "to scale rocprofv3 FETCH_SIZE / WRITE_SIZE readings)")
@@ -192,6 +195,9 @@ def main():
     plan = None
     if not args.no_plan:
         plan = smat_amd.Plan(A["b_row_ptr"], M, K, nnzb, N, col_idx_host=A["b_col_idx"], kernel=args.kernel)
+
+    if plan is not None and not args.no_attach_values:
+        plan.attach_values(vals, rp, ci)  # one-off look at the zero pattern of the blocks (not timed, like the plan)
 
     def step():
         smat_amd.spmm(vals, rp, ci, Bd, Cd, M, N, K, nnzb, plan=plan, kernel=args.kernel)

@@ -68,6 +68,8 @@ int smat_spmm_bcsr_f16(const uint16_t *vals, const int32_t *row_ptr, const int32
                                * the plan decides whether B is first repacked slab-major into scratch   */
 #define SMAT_KERNEL_SWEEP 2   /* workgroup sweeps K for a group of block rows, B panel staged in LDS      */
 #define SMAT_KERNEL_ROWWISE_DIRECT 3 /* row-wise, B always read in place (plan or launch option)          */
+#define SMAT_KERNEL_COMPACT 5  /* only the nonzero columns of the blocks are multiplied (needs
+                               * smat_plan_attach_values); for blocks with few nonzero columns */
 #define SMAT_KERNEL_ROWWISE_PACKED 4 /* row-wise, B always repacked (needs a plan created with this id) */
 
 typedef struct smat_spmm_opts {
@@ -90,10 +92,21 @@ typedef struct smat_plan smat_plan;
  * n_hint: the N the plan will mostly be used with (panel width choice). */
 int smat_plan_create(smat_plan **plan, const int32_t *row_ptr_host, const int32_t *col_idx_host,
                      size_t M, size_t K, size_t nnzb, size_t n_hint, const smat_spmm_opts *opts);
+/* Optional: lets the plan look at the block values (DEVICE arrays of the matrix the plan was
+ * made for; row_ptr_host as in smat_plan_create).  The plan lists the nonzero columns of every
+ * block and keeps a COPY of them (32 bytes per nonzero column, in MFMA operand order), so that
+ * SMAT_KERNEL_COMPACT multiplies only those and touches only the rows of B under them; with
+ * SMAT_KERNEL_AUTO the plan switches to that kernel when fewer than 60% of the block columns
+ * are nonzero.  The compact kernel works from the copy: attach again after the values change.
+ * Synchronous.  No counterpart in the reference, which multiplies every block as a dense
+ * 16x16 (mmaCBT.cu:44-66). */
+int smat_plan_attach_values(smat_plan *plan, const uint16_t *vals, const int32_t *row_ptr,
+                            const int32_t *col_idx, const int32_t *row_ptr_host);
 int smat_plan_destroy(smat_plan *plan);
-/* Fills info[0..8]: kernel id, row-wise work items, split block rows, chunk size,
+/* Fills info[0..9]: kernel id, row-wise work items, split block rows, chunk size,
  * workspace bytes, panel width, sweep MFMA ops, sweep (row group, K chunk) records,
- * bytes of the slab-major scratch copy of B (0 = B is read in place). */
+ * bytes of the scratch copy of B (0 = B is read in place), nonzero block columns listed by
+ * smat_plan_attach_values (0 = not attached). */
 int smat_plan_info(const smat_plan *plan, int64_t *info);
 
 /* Same operands as smat_spmm_bcsr_f16; C is uint16_t* or float* per opts->c_dtype.

@@ -26,6 +26,7 @@ using namespace smat;
 
 struct smat_plan {
     int kernel = SMAT_KERNEL_ROWWISE;
+    int kernel_requested = SMAT_KERNEL_AUTO;
     size_t M = 0, K = 0, nnzb = 0, n_cap = 0;
     int chunk = 0;
     int panel_tiles = 0;
@@ -39,6 +40,9 @@ struct smat_plan {
     int n_rg = 0, n_records = 0, n_ops = 0;
     int32_t *d_rg_chunk_ptr = nullptr, *d_chunk_ids = nullptr;
     SweepOp *d_ops = nullptr;
+    // compacted-column kernel (present after smat_plan_attach_values)
+    CompactPlan *compact = nullptr;
+    uint16_t *d_bt = nullptr; // row-major copy of B, K * n_cap halves (compact kernel)
 };
 
 extern "C" const char *smat_version(void) { return "smat-amd 0.1 gfx950"; }
@@ -100,10 +104,18 @@ extern "C" int smat_spmm_bcsr_f16_ex(const uint16_t *vals, const int32_t *row_pt
     if (kernel == SMAT_KERNEL_ROWWISE_PACKED && !a.b_packed)
         return set_error(SMAT_ERR_INVALID, "SMAT_KERNEL_ROWWISE_PACKED needs a plan built for it with n_hint >= N");
     if (kernel == SMAT_KERNEL_ROWWISE_DIRECT || kernel == SMAT_KERNEL_ROWWISE_PACKED) kernel = SMAT_KERNEL_ROWWISE;
-    if (kernel != SMAT_KERNEL_ROWWISE && kernel != SMAT_KERNEL_SWEEP)
+    if (kernel != SMAT_KERNEL_ROWWISE && kernel != SMAT_KERNEL_SWEEP && kernel != SMAT_KERNEL_COMPACT)
         return set_error(SMAT_ERR_INVALID, "unknown kernel id %d", kernel);
     hipError_t e;
-    if (kernel == SMAT_KERNEL_SWEEP) {
+    if (kernel == SMAT_KERNEL_COMPACT) {
+        if (!plan || !plan->compact || !plan->d_bt || N > plan->n_cap)
+            return set_error(SMAT_ERR_INVALID,
+                             "SMAT_KERNEL_COMPACT needs a plan with attached values (smat_plan_attach_values) and n_hint >= N");
+        CompactArgs c{};
+        c.B = B; c.Bt = plan->d_bt; c.C = C; c.M = M; c.N = N; c.K = K; c.c_f32 = a.c_f32;
+        c.plan = plan->compact;
+        e = launch_compact(c, static_cast<hipStream_t>(o.stream));
+    } else if (kernel == SMAT_KERNEL_SWEEP) {
         if (!plan || !plan->d_ops)
             return set_error(SMAT_ERR_INVALID, "SMAT_KERNEL_SWEEP needs a plan built for it (with col_idx_host)");
         SweepArgs w{};
@@ -157,6 +169,7 @@ extern "C" int smat_plan_create(smat_plan **out, const int32_t *row_ptr_host,
     smat_plan *p = new (std::nothrow) smat_plan();
     if (!p) return set_error(SMAT_ERR_NOMEM, "out of host memory");
     p->M = M; p->K = K; p->nnzb = nnzb; p->n_cap = n_hint;
+    p->kernel_requested = want;
 
     // A block row is split when it is much longer than the average: chunks of
     // `chunk` blocks (even, so block pairs stay aligned with the MFMA K = 32).
@@ -315,9 +328,44 @@ extern "C" int smat_plan_create(smat_plan **out, const int32_t *row_ptr_host,
     return SMAT_OK;
 }
 
+extern "C" int smat_plan_attach_values(smat_plan *p, const uint16_t *vals, const int32_t *row_ptr,
+                                        const int32_t *col_idx, const int32_t *row_ptr_host)
+{
+    if (!p || !row_ptr || !row_ptr_host) return set_error(SMAT_ERR_INVALID, "plan, row_ptr and row_ptr_host must not be NULL");
+    if (p->nnzb && (!vals || !col_idx)) return set_error(SMAT_ERR_INVALID, "vals and col_idx must not be NULL");
+    if (p->compact) { compact_destroy(p->compact); p->compact = nullptr; }
+    CompactPlan *c = nullptr;
+    hipError_t e = compact_build(vals, row_ptr, col_idx, row_ptr_host, p->M / 16, p->nnzb, p->n_cap, &c);
+    if (e != hipSuccess) return set_error(SMAT_ERR_HIP, "attaching values failed: %s", hipGetErrorString(e));
+    // The dense kernels gather 16 rows of B per block, this one a row per nonzero column.  Measured:
+    // 7 nonzero columns per block (27-point stencil) 53 us against 86 us row-wise; 16 per block
+    // (dense blocks, N = 4096) 326 us against 180 us.  The plan's choice below 60% of the columns
+    // (9.6 per block), unless a kernel was asked for.
+    const bool take = p->kernel_requested == SMAT_KERNEL_COMPACT ||
+                      (p->kernel_requested == SMAT_KERNEL_AUTO && (double)c->n_cols < 0.6 * 16.0 * (double)p->nnzb);
+    if (!take) { // nothing will use the list: the plan stays as it was
+        compact_destroy(c);
+        return SMAT_OK;
+    }
+    if (!p->d_bt) e = hipMalloc(&p->d_bt, p->K * p->n_cap * sizeof(uint16_t));
+    if (e != hipSuccess) {
+        compact_destroy(c);
+        return set_error(SMAT_ERR_HIP, "attaching values failed: %s", hipGetErrorString(e));
+    }
+    p->compact = c;
+    p->kernel = SMAT_KERNEL_COMPACT;
+    if (p->d_bpack && p->kernel_requested == SMAT_KERNEL_AUTO) { // the row-wise kernel's scratch is not needed any more
+        (void)hipFree(p->d_bpack);
+        p->d_bpack = nullptr;
+    }
+    return SMAT_OK;
+}
+
 extern "C" int smat_plan_destroy(smat_plan *p)
 {
     if (!p) return SMAT_OK;
+    if (p->compact) compact_destroy(p->compact);
+    if (p->d_bt) (void)hipFree(p->d_bt);
     if (p->d_items) (void)hipFree(p->d_items);
     if (p->d_split) (void)hipFree(p->d_split);
     if (p->d_workspace) (void)hipFree(p->d_workspace);
@@ -336,7 +384,9 @@ extern "C" int smat_plan_info(const smat_plan *p, int64_t *info)
     info[4] = (int64_t)p->workspace_bytes;
     info[5] = p->kernel == SMAT_KERNEL_SWEEP ? 16 * SWEEP_TN : 16 * p->panel_tiles;
     info[6] = p->n_ops; info[7] = p->n_records;
-    info[8] = p->d_bpack ? (int64_t)(p->K * p->n_cap * sizeof(uint16_t)) : 0;
+    info[8] = (p->d_bpack ? (int64_t)(p->K * p->n_cap * sizeof(uint16_t)) : 0) +
+              (p->d_bt ? (int64_t)(p->K * p->n_cap * sizeof(uint16_t)) : 0);
+    info[9] = p->compact ? p->compact->n_cols : 0;
     return SMAT_OK;
 }
 

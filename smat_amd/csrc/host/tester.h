@@ -43,10 +43,15 @@ public:
             smat_spmm_opts o = {SMAT_B_COL_MAJOR, SMAT_C_F16, kernel_, 0, nullptr};
             SMAT_CHECK(smat_plan_create(&plan_, A_->hostBcsrRowPtr(), A_->hostBcsrColIdx(), A_->getRow(), A_->getCol(),
                                         A_->getNonzeroblocks(), N, &o));
-            int64_t info[9];
+            // the plan also looks at the block values once (which columns of the blocks are nonzero)
+            SMAT_CHECK(smat_plan_attach_values(plan_, (const uint16_t *)A_->getBcsrValues(), A_->getBcsrRowPtr(),
+                                               A_->getBcsrColIdx(), A_->hostBcsrRowPtr()));
+            int64_t info[10];
             SMAT_CHECK(smat_plan_info(plan_, info));
-            HLOG("Plan: kernel %lld, %lld work items, %lld split block rows, workspace %lld bytes, %lld sweep ops",
-                 (long long)info[0], (long long)info[1], (long long)info[2], (long long)info[4], (long long)info[6]);
+            HLOG("Plan: kernel %lld, %lld work items, %lld split block rows, workspace %lld bytes, %lld sweep ops, "
+                 "%lld nonzero block columns",
+                 (long long)info[0], (long long)info[1], (long long)info[2], (long long)info[4], (long long)info[6],
+                 (long long)info[9]);
         }
     }
     ~Tester()

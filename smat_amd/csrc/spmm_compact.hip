@@ -1,0 +1,455 @@
+// SpMM for block matrices whose 16x16 blocks hold only a few nonzero COLUMNS (random sparse
+// matrices blocked without much clustering: about one nonzero per block).  The dense kernels
+// gather 16 rows of B for every block; here only the rows of B that meet a nonzero column of A
+// are touched, and 32 such columns of one block row are multiplied per MFMA step.
+//
+// Same product as the reference kernel (src/cuda_hgemm/src/mma/mmaCBT.cu:13-88): an all-zero
+// column of a block contributes nothing to C, so leaving it out changes no result (with finite B).
+//
+//  * compact_build (once per matrix, from the block values):
+//      colmask_kernel   16-bit mask of the nonzero columns of every block (two blocks per
+//                       wavefront step, OR over the 16 rows with cross-lane shuffles);
+//      exclusive scan   of the popcounts; the per-block-row totals go to the host, which pads
+//                       every block row to a multiple of 32 columns (zero columns) and cuts the
+//                       list into work items (whole block rows, long ones in chunks whose fp32
+//                       partial tiles are summed afterwards);
+//      gather_kernel    writes, for every nonzero column, its row of B (absolute column index)
+//                       and a COPY of its 16 values in MFMA operand order:
+//                       acol[((step*4 + g)*16 + m)*8 + j] = A[m][column 32*step + 8*g + j],
+//                       so that the A operand of a step is one coalesced 16-byte load per lane.
+//    The SpMM then does not read the block values any more: they must be attached again when
+//    they change.
+//  * transpose_b_kernel: column-major B (B[n*K + k]) -> row-major Bt[k*N + n] at the start of
+//    every launch, so that the row of B under a nonzero column is contiguous.
+//  * spmm_compact_kernel<TQ>: one wavefront per (work item, panel of 64*TQ columns).  A step takes
+//    32 columns = K of one v_mfma_f32_16x16x32_f16.  The product is formed as
+//    C^T = B^T * A^T like in the other kernels:
+//      A operand   lane (m = lane % 16, g = lane / 16): one 16-byte load from acol;
+//      B operand   lane (i = lane % 16, g) loads 8 bytes = columns 4i .. 4i+3 of row col(entry)
+//                  for each of its 8 entries (16 lanes read 128 contiguous bytes); the q-th
+//                  halves of two consecutive entries are merged with one v_perm_b32 into the
+//                  operand word of n-tile q, so tile q of a 64-column group owns columns 4i + q;
+//      result      lane (m, g) holds rows i = 4g .. 4g+3 of the four tiles = 16 consecutive
+//                  columns of C row m: two 16-byte stores (fp16) per 64-column group.
+#include <hip/hip_runtime.h>
+#include <hipcub/hipcub.hpp>
+#include <stdint.h>
+
+#include <algorithm>
+#include <vector>
+
+#include "spmm_kernels.h"
+
+namespace smat {
+
+typedef _Float16 f16x8 __attribute__((ext_vector_type(8)));
+typedef float f32x4 __attribute__((ext_vector_type(4)));
+typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
+
+namespace {
+
+constexpr int LIST_PAD = 128; // entries readable past the end of the list (the pipeline reads up to three steps ahead)
+
+// ---- census of nonzero block columns ----
+
+__global__ __launch_bounds__(256) void colmask_kernel(const uint16_t *__restrict__ vals, long nnzb,
+                                                      uint16_t *__restrict__ mask, int32_t *__restrict__ count)
+{
+    const int lane = threadIdx.x & 63;
+    const long wave = ((long)blockIdx.x * blockDim.x + threadIdx.x) >> 6;
+    const long n_waves = ((long)gridDim.x * blockDim.x) >> 6;
+    for (long pb = wave * 2; pb < nnzb; pb += n_waves * 2) {
+        const long blk = pb + (lane >> 5);
+        // lane % 32 = row * 2 + half: 8 values of one row
+        u32x4 w = {0u, 0u, 0u, 0u};
+        if (blk < nnzb) w = *reinterpret_cast<const u32x4 *>(vals + blk * 256 + (lane & 31) * 8);
+        w &= 0x7fff7fffu; // -0.0 is a zero
+#pragma unroll
+        for (int d = 2; d <= 16; d <<= 1) { // OR over the 16 rows (lane bits 1..4)
+            w[0] |= __shfl_xor(w[0], d);
+            w[1] |= __shfl_xor(w[1], d);
+            w[2] |= __shfl_xor(w[2], d);
+            w[3] |= __shfl_xor(w[3], d);
+        }
+        uint32_t bits = 0;
+#pragma unroll
+        for (int q = 0; q < 4; q++) {
+            if (w[q] & 0xffffu) bits |= 1u << (2 * q);
+            if (w[q] >> 16) bits |= 1u << (2 * q + 1);
+        }
+        const uint32_t other = __shfl_xor(bits, 1); // the other half of the row
+        if ((lane & 31) == 0 && blk < nnzb) {
+            const uint32_t m = bits | (other << 8);
+            mask[blk] = (uint16_t)m;
+            count[blk] = __popc(m);
+        }
+    }
+}
+
+// One thread per block: its nonzero columns go to positions padded_start[br] + (offset[p] -
+// offset[row_ptr[br]]) .. of the padded list.
+__global__ void gather_kernel(const uint16_t *__restrict__ vals, const uint16_t *__restrict__ mask,
+                              const int32_t *__restrict__ offset, const int32_t *__restrict__ row_ptr,
+                              const int32_t *__restrict__ col_idx, const int32_t *__restrict__ padded_start,
+                              long mb, long nnzb, int32_t *__restrict__ cols, uint16_t *__restrict__ acol)
+{
+    const long p = (long)blockIdx.x * blockDim.x + threadIdx.x;
+    if (p >= nnzb) return;
+    uint32_t m = mask[p];
+    if (!m) return;
+    long lo = 0, hi = mb; // block row of p: largest br with row_ptr[br] <= p
+    while (hi - lo > 1) {
+        const long mid = (lo + hi) >> 1;
+        if (row_ptr[mid] <= p) lo = mid; else hi = mid;
+    }
+    long o = (long)padded_start[lo] + (offset[p] - offset[row_ptr[lo]]);
+    const int32_t c0 = col_idx[p];
+    const uint16_t *blk = vals + p * 256;
+    while (m) {
+        const int k = __ffs(m) - 1;
+        m &= m - 1;
+        cols[o] = c0 + k;
+        uint16_t *dst = acol + ((o >> 3) * 16) * 8 + (o & 7); // (step*4 + g) = o / 8
+#pragma unroll
+        for (int r = 0; r < 16; r++) dst[r * 8] = blk[r * 16 + k];
+        o++;
+    }
+}
+
+// raw[br] = first (unpadded) list position of block row br; raw[mb] = total
+__global__ void row_offsets_kernel(const int32_t *__restrict__ row_ptr, const int32_t *__restrict__ offset,
+                                   const int32_t *__restrict__ count, long mb, long nnzb, int32_t *__restrict__ raw)
+{
+    const long br = (long)blockIdx.x * blockDim.x + threadIdx.x;
+    if (br > mb) return;
+    const long p = row_ptr[br];
+    raw[br] = p < nnzb ? offset[p] : (nnzb ? offset[nnzb - 1] + count[nnzb - 1] : 0);
+}
+
+// ---- B: column-major -> row-major ----
+// 64 n x 64 k tile through LDS.  A thread reads 16 bytes (8 k) of two neighbouring columns, pairs
+// the values of equal k into dwords and writes them to the transposed tile; then every thread
+// reads 8 n of one k back (two 8-byte LDS reads) and stores 16 bytes.
+__global__ __launch_bounds__(256) void transpose_b_kernel(const uint16_t *__restrict__ B, uint16_t *__restrict__ Bt,
+                                                          int N, long K)
+{
+    constexpr int LD = 68; // halfs per LDS row (k): 8-byte aligned rows, dword writes spread over the banks
+    __shared__ __align__(16) uint16_t tile[64 * LD];
+    const int t = threadIdx.x;
+    const long k0 = (long)blockIdx.x * 64;
+    const int n0 = blockIdx.y * 64;
+    {
+        const int np = t >> 3, seg = t & 7; // columns 2np, 2np+1; k = 8seg .. 8seg+7
+        u32x4 v0 = {0u, 0u, 0u, 0u}, v1 = {0u, 0u, 0u, 0u};
+        if (k0 + seg * 8 < K) {
+            if (n0 + 2 * np < N) v0 = *reinterpret_cast<const u32x4 *>(B + (long)(n0 + 2 * np) * K + k0 + seg * 8);
+            if (n0 + 2 * np + 1 < N) v1 = *reinterpret_cast<const u32x4 *>(B + (long)(n0 + 2 * np + 1) * K + k0 + seg * 8);
+        }
+#pragma unroll
+        for (int w = 0; w < 4; w++) {
+            uint32_t *row = reinterpret_cast<uint32_t *>(tile + (seg * 8 + 2 * w) * LD + 2 * np);
+            row[0] = __builtin_amdgcn_perm(v1[w], v0[w], 0x05040100u);      // k = 8seg + 2w
+            row[LD / 2] = __builtin_amdgcn_perm(v1[w], v0[w], 0x07060302u); // k = 8seg + 2w + 1
+        }
+    }
+    __syncthreads();
+    const int a = t >> 3, seg = t & 7;
+#pragma unroll
+    for (int half = 0; half < 2; half++) {
+        const int k = a + 32 * half;
+        if (k0 + k < K && n0 + seg * 8 < N) {
+            const uint2 lo = *reinterpret_cast<const uint2 *>(tile + k * LD + seg * 8);
+            const uint2 hi = *reinterpret_cast<const uint2 *>(tile + k * LD + seg * 8 + 4);
+            *reinterpret_cast<u32x4 *>(Bt + (k0 + k) * (long)N + n0 + seg * 8) = (u32x4){lo.x, lo.y, hi.x, hi.y};
+        }
+    }
+}
+
+// ---- the product ----
+
+template <int TQ, bool C_F32>
+__global__ __launch_bounds__(256) void spmm_compact_kernel(
+    const uint16_t *__restrict__ acol, const int32_t *__restrict__ cols, const uint16_t *__restrict__ Bt,
+    void *__restrict__ Cout, float *__restrict__ workspace, const WorkItem *__restrict__ items, int n_items, int N,
+    int n_panels)
+{
+    constexpr int PANEL = 64 * TQ;
+    const int lane = threadIdx.x & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+    // panel-major order of the (panel, item) space, a contiguous eighth per XCD
+    const long total = (long)n_items * n_panels;
+    const int chunk = gridDim.x >> 3; // gridDim.x is a multiple of 8
+    const long wg = (long)(blockIdx.x & 7) * chunk + (blockIdx.x >> 3);
+    const long w = wg * 4 + wave;
+    if (w >= total) return;
+    const int panel = (int)(w / n_items);
+    const int it = (int)(w - (long)panel * n_items);
+    const WorkItem wi = items[it];
+    const int br = __builtin_amdgcn_readfirstlane(wi.block_row);
+    const int e0 = __builtin_amdgcn_readfirstlane(wi.begin);
+    const int e1 = __builtin_amdgcn_readfirstlane(wi.end);
+    const int dst = __builtin_amdgcn_readfirstlane(wi.dst);
+
+    const int i16 = lane & 15, g = lane >> 4;
+    const int n0 = panel * PANEL;
+    long boff[TQ]; // element offset of this lane's 4 columns inside a row of Bt (column 0 when out of range)
+#pragma unroll
+    for (int q = 0; q < TQ; q++) {
+        const int n = n0 + 64 * q + 4 * i16;
+        boff[q] = n < N ? n : 0; // N % 8 == 0: all four columns or none
+    }
+
+    f32x4 acc[TQ][4];
+#pragma unroll
+    for (int q = 0; q < TQ; q++)
+#pragma unroll
+        for (int t = 0; t < 4; t++) acc[q][t] = (f32x4){0.f, 0.f, 0.f, 0.f};
+
+    // Software pipeline over steps of 32 columns (items start and end on multiples of 32): the
+    // column indices of step s+2, then the operands of step s+1 (whose indices arrived a step
+    // ago) are requested before the MFMAs of step s.  Loads past the end of the item read the
+    // next item's data or the padding behind the arrays: always valid addresses, never used.
+    struct Entries { u32x4 r[2]; };
+    struct Operands { u32x4 aw; uint2 L[TQ][8]; };
+    auto load_entries = [&](int e, Entries &x) {
+        const u32x4 *lp = reinterpret_cast<const u32x4 *>(cols + e + 8 * g);
+        x.r[0] = lp[0]; x.r[1] = lp[1];
+    };
+    auto load_operands = [&](int e, const Entries &x, Operands &o) {
+        const uint32_t col[8] = {x.r[0][0], x.r[0][1], x.r[0][2], x.r[0][3], x.r[1][0], x.r[1][1], x.r[1][2], x.r[1][3]};
+        o.aw = *reinterpret_cast<const u32x4 *>(acol + ((long)(e >> 3) + g) * 128 + i16 * 8);
+#pragma unroll
+        for (int q = 0; q < TQ; q++)
+#pragma unroll
+            for (int j = 0; j < 8; j++)
+                o.L[q][j] = *reinterpret_cast<const uint2 *>(Bt + (long)col[j] * N + boff[q]);
+    };
+    auto multiply = [&](const Operands &o) {
+        const f16x8 av = __builtin_bit_cast(f16x8, o.aw);
+#pragma unroll
+        for (int q = 0; q < TQ; q++) {
+            // tile t of the group takes the t-th of the four columns: words = (entry 2p, entry 2p+1)
+            u32x4 b[4];
+#pragma unroll
+            for (int p = 0; p < 4; p++) {
+                b[0][p] = __builtin_amdgcn_perm(o.L[q][2 * p + 1].x, o.L[q][2 * p].x, 0x05040100u);
+                b[1][p] = __builtin_amdgcn_perm(o.L[q][2 * p + 1].x, o.L[q][2 * p].x, 0x07060302u);
+                b[2][p] = __builtin_amdgcn_perm(o.L[q][2 * p + 1].y, o.L[q][2 * p].y, 0x05040100u);
+                b[3][p] = __builtin_amdgcn_perm(o.L[q][2 * p + 1].y, o.L[q][2 * p].y, 0x07060302u);
+            }
+#pragma unroll
+            for (int t = 0; t < 4; t++)
+                acc[q][t] = __builtin_amdgcn_mfma_f32_16x16x32_f16(__builtin_bit_cast(f16x8, b[t]), av, acc[q][t], 0, 0, 0);
+        }
+    };
+    if (e0 < e1) {
+        Entries ent_a, ent_b;
+        Operands op_a, op_b;
+        load_entries(e0, ent_a);
+        load_entries(e0 + 32, ent_b);
+        load_operands(e0, ent_a, op_a);
+        int e = e0;
+        while (true) {
+            load_entries(e + 64, ent_a);
+            load_operands(e + 32, ent_b, op_b);
+            multiply(op_a);
+            e += 32;
+            if (e >= e1) break;
+            load_entries(e + 64, ent_b);
+            load_operands(e + 32, ent_a, op_a);
+            multiply(op_b);
+            e += 32;
+            if (e >= e1) break;
+        }
+    }
+
+    // acc[q][t][r] = C[br*16 + i16][n0 + 64q + 16g + 4r + t]
+    const long m = (long)br * 16 + i16;
+#pragma unroll
+    for (int q = 0; q < TQ; q++) {
+        const int c0 = n0 + 64 * q + 16 * g;
+        float o[16];
+#pragma unroll
+        for (int r = 0; r < 4; r++)
+#pragma unroll
+            for (int t = 0; t < 4; t++) o[4 * r + t] = acc[q][t][r];
+        if (dst >= 0 || C_F32) {
+            float *row = dst >= 0 ? workspace + ((long)dst * 16 + i16) * (long)N
+                                  : reinterpret_cast<float *>(Cout) + m * (long)N;
+#pragma unroll
+            for (int h = 0; h < 4; h++)
+                if (c0 + 4 * h < N)
+                    *reinterpret_cast<f32x4 *>(row + c0 + 4 * h) = (f32x4){o[4 * h], o[4 * h + 1], o[4 * h + 2], o[4 * h + 3]};
+        } else {
+            uint16_t *row = reinterpret_cast<uint16_t *>(Cout) + m * (long)N;
+#pragma unroll
+            for (int h = 0; h < 2; h++) {
+                f16x8 v;
+#pragma unroll
+                for (int j = 0; j < 8; j++) v[j] = (_Float16)o[8 * h + j];
+                if (c0 + 8 * h < N) *reinterpret_cast<f16x8 *>(row + c0 + 8 * h) = v;
+            }
+        }
+    }
+}
+
+template <int TQ>
+hipError_t launch_compact_tq(const CompactArgs &a, hipStream_t st)
+{
+    const CompactPlan &p = *a.plan;
+    const int n_panels = (int)((a.N + 64 * TQ - 1) / (64 * TQ));
+    const long total = (long)p.n_items * n_panels;
+    long wgs = (total + 3) / 4;
+    wgs = (wgs + 7) / 8 * 8;
+    if (wgs == 0) return hipSuccess;
+    if (wgs > 0x7fffffffL) return hipErrorInvalidValue;
+    if (a.c_f32)
+        hipLaunchKernelGGL((spmm_compact_kernel<TQ, true>), dim3((unsigned)wgs), dim3(256), 0, st, p.d_acol, p.d_cols,
+                           a.Bt, a.C, p.d_workspace, p.d_items, p.n_items, (int)a.N, n_panels);
+    else
+        hipLaunchKernelGGL((spmm_compact_kernel<TQ, false>), dim3((unsigned)wgs), dim3(256), 0, st, p.d_acol, p.d_cols,
+                           a.Bt, a.C, p.d_workspace, p.d_items, p.n_items, (int)a.N, n_panels);
+    return hipGetLastError();
+}
+
+struct Scratch {
+    void *p = nullptr;
+    ~Scratch() { if (p) (void)hipFree(p); }
+    hipError_t alloc(size_t bytes) { return hipMalloc(&p, bytes ? bytes : 16); }
+};
+
+} // namespace
+
+hipError_t launch_compact(const CompactArgs &a, hipStream_t st)
+{
+    dim3 grid((unsigned)((a.K + 63) / 64), (unsigned)((a.N + 63) / 64));
+    hipLaunchKernelGGL(transpose_b_kernel, grid, dim3(256), 0, st, a.B, a.Bt, (int)a.N, (long)a.K);
+    hipError_t e = hipGetLastError();
+    if (e != hipSuccess) return e;
+    // wide panels reuse the A operand over more columns; narrow ones give more wavefronts
+    const long items = a.plan->n_items;
+    if (a.N >= 256 && items * (long)(a.N / 256) >= 4096) e = launch_compact_tq<4>(a, st);
+    else if (a.N >= 128 && items * (long)(a.N / 128) >= 2048) e = launch_compact_tq<2>(a, st);
+    else e = launch_compact_tq<1>(a, st);
+    if (e != hipSuccess) return e;
+    if (a.plan->n_split_rows > 0)
+        e = launch_reduce(a.plan->d_workspace, a.plan->d_split, a.plan->n_split_rows, a.C, a.N, a.c_f32, st);
+    return e;
+}
+
+void compact_destroy(CompactPlan *p)
+{
+    if (!p) return;
+    if (p->d_cols) (void)hipFree(p->d_cols);
+    if (p->d_acol) (void)hipFree(p->d_acol);
+    if (p->d_items) (void)hipFree(p->d_items);
+    if (p->d_split) (void)hipFree(p->d_split);
+    if (p->d_workspace) (void)hipFree(p->d_workspace);
+    delete p;
+}
+
+hipError_t compact_build(const uint16_t *vals, const int32_t *row_ptr, const int32_t *col_idx,
+                         const int32_t *row_ptr_host, size_t mb, size_t nnzb, size_t n_cap, CompactPlan **out)
+{
+    *out = nullptr;
+    CompactPlan *p = new (std::nothrow) CompactPlan();
+    if (!p) return hipErrorOutOfMemory;
+    hipError_t e = hipSuccess;
+    Scratch mask, count, offset, tmp, cc;
+#define SMAT_STEP(call)                                                                            \
+    do {                                                                                           \
+        if (e == hipSuccess) e = (call);                                                           \
+    } while (0)
+    SMAT_STEP(mask.alloc(nnzb * 2));
+    SMAT_STEP(count.alloc(nnzb * 4));
+    SMAT_STEP(offset.alloc(nnzb * 4));
+    SMAT_STEP(cc.alloc((mb + 1) * 4));
+    int64_t n_cols = 0;
+    std::vector<int32_t> raw(mb + 1, 0), padded(mb + 1, 0);
+    if (e == hipSuccess && nnzb) {
+        const long waves = std::min<long>((long)(nnzb + 1) / 2, 256L * 32);
+        hipLaunchKernelGGL(colmask_kernel, dim3((unsigned)((waves + 3) / 4)), dim3(256), 0, 0, vals, (long)nnzb,
+                           (uint16_t *)mask.p, (int32_t *)count.p);
+        e = hipGetLastError();
+        size_t bytes = 0;
+        SMAT_STEP(hipcub::DeviceScan::ExclusiveSum(nullptr, bytes, (int32_t *)count.p, (int32_t *)offset.p, (int)nnzb));
+        SMAT_STEP(tmp.alloc(bytes));
+        SMAT_STEP(hipcub::DeviceScan::ExclusiveSum(tmp.p, bytes, (int32_t *)count.p, (int32_t *)offset.p, (int)nnzb));
+        if (e == hipSuccess) {
+            hipLaunchKernelGGL(row_offsets_kernel, dim3((unsigned)((mb + 1 + 255) / 256)), dim3(256), 0, 0, row_ptr,
+                               (const int32_t *)offset.p, (const int32_t *)count.p, (long)mb, (long)nnzb, (int32_t *)cc.p);
+            e = hipGetLastError();
+        }
+        SMAT_STEP(hipMemcpy(raw.data(), cc.p, (mb + 1) * 4, hipMemcpyDeviceToHost));
+        n_cols = raw[mb];
+    }
+    p->n_cols = n_cols;
+    // every block row is padded to a multiple of 32 columns (one MFMA step); padding = zero columns
+    int64_t total = 0;
+    for (size_t i = 0; i < mb; i++) {
+        padded[i] = (int32_t)total;
+        total += ((int64_t)(raw[i + 1] - raw[i]) + 31) / 32 * 32;
+        if (total > 0x7fffff00) e = hipErrorInvalidValue;
+    }
+    padded[mb] = (int32_t)total;
+    const size_t cap = (size_t)total + LIST_PAD;
+    SMAT_STEP(hipMalloc(&p->d_cols, cap * sizeof(int32_t)));
+    SMAT_STEP(hipMemset(p->d_cols, 0, cap * sizeof(int32_t))); // padding: row 0 of B
+    SMAT_STEP(hipMalloc(&p->d_acol, cap * 16 * sizeof(uint16_t)));
+    SMAT_STEP(hipMemset(p->d_acol, 0, cap * 16 * sizeof(uint16_t)));
+    if (e == hipSuccess && nnzb) {
+        SMAT_STEP(hipMemcpy(cc.p, padded.data(), (mb + 1) * 4, hipMemcpyHostToDevice));
+        if (e == hipSuccess) {
+            hipLaunchKernelGGL(gather_kernel, dim3((unsigned)((nnzb + 255) / 256)), dim3(256), 0, 0, vals,
+                               (const uint16_t *)mask.p, (const int32_t *)offset.p, row_ptr, col_idx,
+                               (const int32_t *)cc.p, (long)mb, (long)nnzb, p->d_cols, p->d_acol);
+            e = hipGetLastError();
+        }
+    }
+    // work items: whole block rows; rows much longer than the average in chunks of 32-column steps
+    (void)row_ptr_host;
+    const std::vector<int32_t> &cc_host = padded;
+    size_t nonempty = 0;
+    for (size_t i = 0; i < mb; i++) nonempty += cc_host[i + 1] > cc_host[i];
+    const double avg = nonempty ? (double)total / (double)nonempty : 0.0;
+    long chunk = (long)(4.0 * avg + 0.5);
+    chunk = std::max(chunk, 512L);
+    chunk = (chunk + 31) / 32 * 32;
+    std::vector<WorkItem> items;
+    std::vector<SplitRow> split;
+    int slot = 0;
+    for (size_t i = 0; i < mb; i++) {
+        const long len = cc_host[i + 1] - cc_host[i];
+        if (len <= chunk) continue;
+        SplitRow sr{(int32_t)i, slot, slot, 0};
+        for (long b = cc_host[i]; b < cc_host[i + 1]; b += chunk)
+            items.push_back(WorkItem{(int32_t)i, (int32_t)b, (int32_t)std::min<long>(b + chunk, cc_host[i + 1]), slot++});
+        sr.slot_end = slot;
+        split.push_back(sr);
+    }
+    for (size_t i = 0; i < mb; i++) {
+        const long len = cc_host[i + 1] - cc_host[i];
+        if (len > chunk) continue;
+        items.push_back(WorkItem{(int32_t)i, cc_host[i], cc_host[i + 1], -1});
+    }
+    p->n_items = (int)items.size();
+    p->n_split_rows = (int)split.size();
+    p->n_slots = slot;
+    SMAT_STEP(hipMalloc(&p->d_items, std::max<size_t>(items.size(), 1) * sizeof(WorkItem)));
+    if (!items.empty()) SMAT_STEP(hipMemcpy(p->d_items, items.data(), items.size() * sizeof(WorkItem), hipMemcpyHostToDevice));
+    if (!split.empty()) {
+        SMAT_STEP(hipMalloc(&p->d_split, split.size() * sizeof(SplitRow)));
+        SMAT_STEP(hipMemcpy(p->d_split, split.data(), split.size() * sizeof(SplitRow), hipMemcpyHostToDevice));
+        SMAT_STEP(hipMalloc(&p->d_workspace, (size_t)slot * 16 * n_cap * sizeof(float)));
+    }
+    SMAT_STEP(hipDeviceSynchronize());
+#undef SMAT_STEP
+    if (e != hipSuccess) {
+        compact_destroy(p);
+        return e;
+    }
+    *out = p;
+    return hipSuccess;
+}
+
+} // namespace smat

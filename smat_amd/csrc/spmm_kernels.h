@@ -76,6 +76,36 @@ struct SweepArgs {
     int n_rg;
 };
 
+// Sums the fp32 partial tiles of split block rows (workspace[(slot*16 + i)*N + n]) in slot order.
+hipError_t launch_reduce(const float *workspace, const SplitRow *split_rows, int n_split_rows, void *C, size_t N,
+                         bool c_f32, hipStream_t st);
+
+// ---- compacted-column kernel (spmm_compact.hip) ----
+// For matrices whose blocks hold only a few nonzero columns: the nonzero columns of a block
+// row are listed once (from the zero pattern of the values) and multiplied 32 at a time.
+struct CompactPlan {
+    int32_t *d_cols = nullptr;   // row of B (absolute column of A) of every listed column; block rows padded to 32
+    uint16_t *d_acol = nullptr;  // the 16 values of every listed column, in MFMA operand order (32 bytes per column)
+    WorkItem *d_items = nullptr; // begin/end index the padded list
+    SplitRow *d_split = nullptr;
+    float *d_workspace = nullptr; // n_slots * 16 * n_cap floats
+    int n_items = 0, n_split_rows = 0, n_slots = 0;
+    int64_t n_cols = 0;           // nonzero block columns (without padding)
+};
+// vals / row_ptr / col_idx: device BCSR arrays; row_ptr_host: host copy of row_ptr.
+hipError_t compact_build(const uint16_t *vals, const int32_t *row_ptr, const int32_t *col_idx,
+                         const int32_t *row_ptr_host, size_t mb, size_t nnzb, size_t n_cap, CompactPlan **out);
+void compact_destroy(CompactPlan *p);
+struct CompactArgs {
+    const uint16_t *B; // column-major
+    uint16_t *Bt;      // scratch, K * N halves: row-major copy of B made at the start of the launch
+    void *C;
+    size_t M, N, K;
+    bool c_f32;
+    const CompactPlan *plan;
+};
+hipError_t launch_compact(const CompactArgs &a, hipStream_t st);
+
 int rowwise_panel_tiles(size_t N, int requested, size_t n_items);
 hipError_t launch_sweep(const SweepArgs &a, hipStream_t st);
 hipError_t launch_rowwise(const SpmmArgs &a, hipStream_t st);

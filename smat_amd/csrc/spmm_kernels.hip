@@ -326,19 +326,24 @@ hipError_t launch_rowwise(const SpmmArgs &a, hipStream_t st)
     default: e = launch_rowwise_tn<1>(a, st); break;
     }
     if (e != hipSuccess) return e;
-    if (a.n_split_rows > 0) {
-        const long threads = (long)a.n_split_rows * 16 * (long)(a.N / 4);
-        const long blocks = (threads + 255) / 256;
-        if (blocks > 0x7fffffffL) return hipErrorInvalidValue;
-        if (a.c_f32)
-            hipLaunchKernelGGL((spmm_reduce_kernel<true>), dim3((unsigned)blocks), dim3(256), 0, st,
-                               a.workspace, a.split_rows, a.n_split_rows, a.C, (int)a.N);
-        else
-            hipLaunchKernelGGL((spmm_reduce_kernel<false>), dim3((unsigned)blocks), dim3(256), 0, st,
-                               a.workspace, a.split_rows, a.n_split_rows, a.C, (int)a.N);
-        e = hipGetLastError();
-    }
+    if (a.n_split_rows > 0) e = launch_reduce(a.workspace, a.split_rows, a.n_split_rows, a.C, a.N, a.c_f32, st);
     return e;
+}
+
+hipError_t launch_reduce(const float *workspace, const SplitRow *split_rows, int n_split_rows, void *C, size_t N,
+                         bool c_f32, hipStream_t st)
+{
+    const long threads = (long)n_split_rows * 16 * (long)(N / 4);
+    const long blocks = (threads + 255) / 256;
+    if (blocks <= 0) return hipSuccess;
+    if (blocks > 0x7fffffffL) return hipErrorInvalidValue;
+    if (c_f32)
+        hipLaunchKernelGGL((spmm_reduce_kernel<true>), dim3((unsigned)blocks), dim3(256), 0, st, workspace,
+                           split_rows, n_split_rows, C, (int)N);
+    else
+        hipLaunchKernelGGL((spmm_reduce_kernel<false>), dim3((unsigned)blocks), dim3(256), 0, st, workspace,
+                           split_rows, n_split_rows, C, (int)N);
+    return hipGetLastError();
 }
 
 } // namespace smat

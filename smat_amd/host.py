@@ -11,7 +11,7 @@ import numpy as np
 from ._lib import SpmmOpts, check, lib
 
 BS = 16
-KERNEL_AUTO, KERNEL_ROWWISE, KERNEL_SWEEP, KERNEL_ROWWISE_DIRECT, KERNEL_ROWWISE_PACKED = 0, 1, 2, 3, 4
+KERNEL_AUTO, KERNEL_ROWWISE, KERNEL_SWEEP, KERNEL_ROWWISE_DIRECT, KERNEL_ROWWISE_PACKED, KERNEL_COMPACT = 0, 1, 2, 3, 4, 5
 C_F16, C_F32 = 0, 1
 
 
@@ -215,16 +215,22 @@ class Plan:
         ci = None if col_idx_host is None else np.ascontiguousarray(col_idx_host, dtype=np.int32)
         opts = SpmmOpts(0, 0, kernel, 0, None)
         check(lib.smat_plan_create(C.byref(self._h), _p(rp), _p(ci), M, K, nnzb, n_hint, C.byref(opts)))
+        self._rp_host = rp
+
+    def attach_values(self, vals_dev, row_ptr_dev, col_idx_dev):
+        """Let the plan list the nonzero columns of the blocks (device tensors of the same matrix)."""
+        ptr = lambda t: C.c_void_p(t.data_ptr()) if t is not None else None  # noqa: E731
+        check(lib.smat_plan_attach_values(self._h, ptr(vals_dev), ptr(row_ptr_dev), ptr(col_idx_dev), _p(self._rp_host)))
 
     @property
     def handle(self):
         return self._h
 
     def info(self):
-        out = (C.c_int64 * 9)()
+        out = (C.c_int64 * 10)()
         check(lib.smat_plan_info(self._h, out))
         keys = ("kernel", "items", "split_rows", "chunk", "workspace_bytes", "panel", "sweep_ops", "sweep_records",
-                "b_pack_bytes")
+                "b_pack_bytes", "compact_cols")
         return dict(zip(keys, out))
 
     def close(self):

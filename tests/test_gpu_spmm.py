@@ -295,3 +295,78 @@ def test_config4_block_pruned_full_size_sampled_rows(smat, cuda, oracle):
     assert oracle.compare(got3, ref)[0] <= TOL_F16
     d = np.abs(C3.view(np.float16).astype(np.float32) - C.view(np.float16).astype(np.float32)).max()
     assert d <= 2e-3 * np.abs(C.view(np.float16).astype(np.float32)).max()
+
+
+COMPACT = 5
+
+
+def gpu_spmm_compact(smat, cuda, A, B_bits, N, c_f32=False, kernel=COMPACT, n_hint=None):
+    """SpMM through a plan that has looked at the zero pattern of the values."""
+    import torch
+    M, K, nnzb = A["M"], A["K"], int(A["b_col_idx"].shape[0])
+    vals = to_dev(torch, A["b_val"] if nnzb else np.zeros(8, np.uint16), cuda)
+    rp = to_dev(torch, A["b_row_ptr"].astype(np.int32), cuda)
+    ci = to_dev(torch, A["b_col_idx"].astype(np.int32) if nnzb else np.zeros(1, np.int32), cuda)
+    B = to_dev(torch, B_bits, cuda)
+    C = torch.full((M, N), float("nan"), dtype=torch.float32, device=cuda) if c_f32 else \
+        torch.full((M, N), 0x7E00, dtype=torch.int16, device=cuda)
+    p = smat.Plan(A["b_row_ptr"], M, K, nnzb, n_hint or N, col_idx_host=A["b_col_idx"], kernel=kernel)
+    p.attach_values(vals, rp, ci)
+    info = p.info()
+    smat.spmm(vals, rp, ci, B, C, M, N, K, nnzb, plan=p, c_f32=c_f32, kernel=kernel)
+    torch.cuda.synchronize()
+    out = C.cpu().numpy()
+    p.close()
+    return (out if c_f32 else out.view(np.uint16)), info
+
+
+def bcsr_of(smat, d):
+    b = smat.csr_to_bcsr(d["M"], d["K"], d["row_ptr"], d["col_idx"], d["val"])
+    return {"M": b.M, "K": b.K, "b_row_ptr": b.row_ptr, "b_col_idx": b.col_idx, "b_val": b.val, "nnzb": b.nnzb}
+
+
+@pytest.mark.parametrize("N", [8, 64, 72, 128, 264, 520])
+def test_compact_kernel_sparse_blocks(smat, cuda, oracle, N):
+    d = gen.erdos_renyi(1024, 0.004, seed=31 + N)          # about one nonzero per block
+    A = bcsr_of(smat, d)
+    B = gen.dense_b(A["K"], N, seed=N + 11, dist="normal")
+    ref = oracle_ref(oracle, A, B, N)
+    C, info = gpu_spmm_compact(smat, cuda, A, B, N)
+    nz_cols = len(set(zip((np.repeat(np.arange(d["M"]), np.diff(d["row_ptr"])) // 16).tolist(), d["col_idx"].tolist())))
+    assert info["compact_cols"] == nz_cols                  # one list entry per nonzero (block row, column)
+    assert oracle.compare(C, ref)[0] <= TOL_F16
+    C32, _ = gpu_spmm_compact(smat, cuda, A, B, N, c_f32=True)
+    assert rel_err_f32(C32, ref) <= TOL_F32
+    assert np.array_equal(C32.astype(np.float16).view(np.uint16), C)
+
+
+def test_compact_kernel_dense_blocks_split_rows_and_auto(smat, cuda, oracle):
+    # dense blocks (every column nonzero), one very long block row (split into chunks), empty rows
+    lengths = [0, 300, 1, 0, 2, 0, 0, 7] + [3] * 24
+    A = gen.random_bcsr(len(lengths), 320, 0.0, seed=6, row_lengths=lengths)
+    N = 136
+    B = gen.dense_b(A["K"], N, seed=2)
+    ref = oracle_ref(oracle, A, B, N)
+    C, info = gpu_spmm_compact(smat, cuda, A, B, N)
+    assert info["compact_cols"] == 16 * A["nnzb"]
+    assert oracle.compare(C, ref)[0] <= TOL_F16
+    assert not C.reshape(A["M"], N)[0:16].any()
+    # with SMAT_KERNEL_AUTO the plan keeps a dense kernel for dense blocks and takes the compact one for sparse blocks
+    _, info_auto = gpu_spmm_compact(smat, cuda, A, B, N, kernel=0)
+    assert info_auto["kernel"] != COMPACT
+    d = gen.rmat(11, 8, seed=3)
+    As = bcsr_of(smat, d)
+    Bs = gen.dense_b(As["K"], 128, seed=4, dist="uniform")
+    Cs, info_s = gpu_spmm_compact(smat, cuda, As, Bs, 128, kernel=0, n_hint=256)
+    assert info_s["kernel"] == COMPACT
+    assert oracle.compare(Cs, oracle_ref(oracle, As, Bs, 128))[0] <= TOL_F16
+
+
+def test_compact_kernel_needs_attached_values(smat, cuda):
+    import torch
+    A = gen.random_bcsr(4, 4, 0.5, seed=1)
+    p = smat.Plan(A["b_row_ptr"], A["M"], A["K"], A["nnzb"], 64, col_idx_host=A["b_col_idx"])
+    t = torch.zeros(A["M"] * 64, dtype=torch.int16, device=cuda)
+    with pytest.raises(smat.SmatError, match="attach"):
+        smat.spmm(t, t, t, t, t, A["M"], 64, A["K"], A["nnzb"], plan=p, kernel=COMPACT)
+    p.close()
