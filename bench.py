@@ -52,9 +52,16 @@ def build_workload(name):
         b = smat_amd.csr_to_bcsr(d["M"], d["K"], d["row_ptr"], d["col_idx"], d["val"])
         A = {"M": b.M, "K": b.K, "b_row_ptr": b.row_ptr, "b_col_idx": b.col_idx, "b_val": b.val, "nnzb": b.nnzb}
         N, bdist, bseed = 128, "uniform", 0xB0000001
-    elif name == "stencil27_64_N64":
+    elif name in ("stencil27_64_N64", "stencil27_64_reordered_N64"):
         d = gen.stencil27(64)
         b = smat_amd.csr_to_bcsr(d["M"], d["K"], d["row_ptr"], d["col_idx"], d["val"])
+        if "reordered" in name:
+            t0 = time.perf_counter()
+            pr, pc, _, _ = smat_amd.reorder_csr(d["M"], d["K"], d["row_ptr"], d["col_idx"], 16, 16, 0.5, True)
+            INFO["reorder_s"] = round(time.perf_counter() - t0, 3)
+            INFO["nnzb_before_reorder"] = int(b.nnzb)
+            rp, ci, v = smat_amd.permute_csr(d["M"], d["K"], d["row_ptr"], d["col_idx"], d["val"], pr, pc)
+            b = smat_amd.csr_to_bcsr(d["M"], d["K"], rp, ci, v)
         A = {"M": b.M, "K": b.K, "b_row_ptr": b.row_ptr, "b_col_idx": b.col_idx, "b_val": b.val, "nnzb": b.nnzb}
         N, bdist, bseed = 64, "uniform", 0xB0000005
     elif name in ("er_16384_0.1pct_N256", "er_16384_0.1pct_reordered_N256"):

@@ -60,6 +60,8 @@ int smat_spmm_bcsr_f16(const uint16_t *vals, const int32_t *row_ptr, const int32
 
 /* ---- SpMM with options / explicit stream / plan -------------------------- */
 #define SMAT_B_COL_MAJOR 0 /* B[n*K + k]: the reference layout               */
+#define SMAT_B_ROW_MAJOR 1 /* B[k*N + n]: SMAT_KERNEL_COMPACT only (it reads rows of B; column-major B
+                            * is first copied row-major into plan scratch on every launch) */
 #define SMAT_C_F16 0       /* the reference output type                      */
 #define SMAT_C_F32 1       /* keep the fp32 accumulators                     */
 
@@ -73,7 +75,7 @@ int smat_spmm_bcsr_f16(const uint16_t *vals, const int32_t *row_ptr, const int32
 #define SMAT_KERNEL_ROWWISE_PACKED 4 /* row-wise, B always repacked (needs a plan created with this id) */
 
 typedef struct smat_spmm_opts {
-    int32_t b_layout; /* SMAT_B_COL_MAJOR                                   */
+    int32_t b_layout; /* SMAT_B_COL_MAJOR | SMAT_B_ROW_MAJOR                */
     int32_t c_dtype;  /* SMAT_C_F16 | SMAT_C_F32                            */
     int32_t kernel;   /* SMAT_KERNEL_*                                      */
     int32_t reserved; /* must be 0                                          */

@@ -74,8 +74,8 @@ extern "C" int smat_spmm_bcsr_f16_ex(const uint16_t *vals, const int32_t *row_pt
     if (rc) return rc;
     smat_spmm_opts o = {SMAT_B_COL_MAJOR, SMAT_C_F16, SMAT_KERNEL_AUTO, 0, nullptr};
     if (opts) o = *opts;
-    if (o.b_layout != SMAT_B_COL_MAJOR)
-        return set_error(SMAT_ERR_UNSUPPORTED, "only column-major B (B[n*K+k]) is implemented");
+    if (o.b_layout != SMAT_B_COL_MAJOR && o.b_layout != SMAT_B_ROW_MAJOR)
+        return set_error(SMAT_ERR_INVALID, "b_layout must be SMAT_B_COL_MAJOR or SMAT_B_ROW_MAJOR");
     if (o.c_dtype != SMAT_C_F16 && o.c_dtype != SMAT_C_F32)
         return set_error(SMAT_ERR_INVALID, "c_dtype must be SMAT_C_F16 or SMAT_C_F32");
     if (o.c_dtype == SMAT_C_F32 && (reinterpret_cast<uintptr_t>(C) & 15))
@@ -107,12 +107,16 @@ extern "C" int smat_spmm_bcsr_f16_ex(const uint16_t *vals, const int32_t *row_pt
     if (kernel != SMAT_KERNEL_ROWWISE && kernel != SMAT_KERNEL_SWEEP && kernel != SMAT_KERNEL_COMPACT)
         return set_error(SMAT_ERR_INVALID, "unknown kernel id %d", kernel);
     hipError_t e;
+    if (o.b_layout == SMAT_B_ROW_MAJOR && kernel != SMAT_KERNEL_COMPACT)
+        return set_error(SMAT_ERR_UNSUPPORTED,
+                         "row-major B (B[k*N+n]) is implemented for SMAT_KERNEL_COMPACT only; the other kernels "
+                         "take the reference layout B[n*K+k]");
     if (kernel == SMAT_KERNEL_COMPACT) {
         if (!plan || !plan->compact || !plan->d_bt || N > plan->n_cap)
             return set_error(SMAT_ERR_INVALID,
                              "SMAT_KERNEL_COMPACT needs a plan with attached values (smat_plan_attach_values) and n_hint >= N");
         CompactArgs c{};
-        c.B = B; c.Bt = plan->d_bt; c.C = C; c.M = M; c.N = N; c.K = K; c.c_f32 = a.c_f32;
+        c.B = B; c.Bt = plan->d_bt; c.b_row_major = o.b_layout == SMAT_B_ROW_MAJOR; c.C = C; c.M = M; c.N = N; c.K = K; c.c_f32 = a.c_f32;
         c.plan = plan->compact;
         e = launch_compact(c, static_cast<hipStream_t>(o.stream));
     } else if (kernel == SMAT_KERNEL_SWEEP) {

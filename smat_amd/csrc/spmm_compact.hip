@@ -320,12 +320,18 @@ struct Scratch {
 
 } // namespace
 
-hipError_t launch_compact(const CompactArgs &a, hipStream_t st)
+hipError_t launch_compact(const CompactArgs &a_in, hipStream_t st)
 {
-    dim3 grid((unsigned)((a.K + 63) / 64), (unsigned)((a.N + 63) / 64));
-    hipLaunchKernelGGL(transpose_b_kernel, grid, dim3(256), 0, st, a.B, a.Bt, (int)a.N, (long)a.K);
-    hipError_t e = hipGetLastError();
-    if (e != hipSuccess) return e;
+    CompactArgs a = a_in;
+    hipError_t e = hipSuccess;
+    if (a.b_row_major) {
+        a.Bt = const_cast<uint16_t *>(a.B); // read in place, never written
+    } else {
+        dim3 grid((unsigned)((a.K + 63) / 64), (unsigned)((a.N + 63) / 64));
+        hipLaunchKernelGGL(transpose_b_kernel, grid, dim3(256), 0, st, a.B, a.Bt, (int)a.N, (long)a.K);
+        e = hipGetLastError();
+        if (e != hipSuccess) return e;
+    }
     // wide panels reuse the A operand over more columns; narrow ones give more wavefronts
     const long items = a.plan->n_items;
     if (a.N >= 256 && items * (long)(a.N / 256) >= 4096) e = launch_compact_tq<4>(a, st);

@@ -97,7 +97,8 @@ hipError_t compact_build(const uint16_t *vals, const int32_t *row_ptr, const int
                          const int32_t *row_ptr_host, size_t mb, size_t nnzb, size_t n_cap, CompactPlan **out);
 void compact_destroy(CompactPlan *p);
 struct CompactArgs {
-    const uint16_t *B; // column-major
+    const uint16_t *B; // column-major, or row-major with b_row_major
+    bool b_row_major;  // B is already B[k*N + n]: no copy is made
     uint16_t *Bt;      // scratch, K * N halves: row-major copy of B made at the start of the launch
     void *C;
     size_t M, N, K;

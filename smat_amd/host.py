@@ -246,7 +246,7 @@ class Plan:
 
 
 def spmm(vals, row_ptr, col_idx, B, C_out, M, N, K, nnzb, plan=None, c_f32=False, kernel=KERNEL_AUTO,
-         stream=None, drop_in=False):
+         stream=None, drop_in=False, b_row_major=False):
     """Launch the SpMM on device tensors (anything with .data_ptr()).
 
     drop_in=True calls the positional drop-in entry point (smat_spmm_bcsr_f16) with
@@ -256,6 +256,7 @@ def spmm(vals, row_ptr, col_idx, B, C_out, M, N, K, nnzb, plan=None, c_f32=False
         check(lib.smat_spmm_bcsr_f16(ptr(vals), ptr(row_ptr), ptr(col_idx), ptr(B), ptr(C_out), M, N, K, nnzb,
                                      None, None))
         return
-    opts = SpmmOpts(0, C_F32 if c_f32 else C_F16, kernel, 0, C.c_void_p(stream) if stream else None)
+    opts = SpmmOpts(1 if b_row_major else 0, C_F32 if c_f32 else C_F16, kernel, 0,
+                    C.c_void_p(stream) if stream else None)
     check(lib.smat_spmm_bcsr_f16_ex(ptr(vals), ptr(row_ptr), ptr(col_idx), ptr(B), ptr(C_out), M, N, K, nnzb,
                                     C.byref(opts), plan.handle if plan is not None else None))

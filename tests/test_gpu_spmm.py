@@ -370,3 +370,29 @@ def test_compact_kernel_needs_attached_values(smat, cuda):
     with pytest.raises(smat.SmatError, match="attach"):
         smat.spmm(t, t, t, t, t, A["M"], 64, A["K"], A["nnzb"], plan=p, kernel=COMPACT)
     p.close()
+
+
+def test_compact_kernel_row_major_b(smat, cuda, oracle):
+    """Row-major B (B[k*N + n]) skips the per-launch copy: same bits as with the reference layout."""
+    import torch
+    d = gen.erdos_renyi(2048, 0.003, seed=8)
+    A = bcsr_of(smat, d)
+    N = 200
+    B = gen.dense_b(A["K"], N, seed=5, dist="normal")                      # column-major bits
+    B_rm = np.ascontiguousarray(B.reshape(N, A["K"]).T).ravel()           # the same matrix, row-major
+    M, K, nnzb = A["M"], A["K"], A["nnzb"]
+    vals, rp, ci = to_dev(torch, A["b_val"], cuda), to_dev(torch, A["b_row_ptr"], cuda), to_dev(torch, A["b_col_idx"], cuda)
+    p = smat.Plan(A["b_row_ptr"], M, K, nnzb, N, col_idx_host=A["b_col_idx"], kernel=COMPACT)
+    p.attach_values(vals, rp, ci)
+    out = []
+    for bits, rm in ((B, False), (B_rm, True)):
+        C = torch.full((M, N), 0x7E00, dtype=torch.int16, device=cuda)
+        smat.spmm(vals, rp, ci, to_dev(torch, bits, cuda), C, M, N, K, nnzb, plan=p, kernel=COMPACT, b_row_major=rm)
+        torch.cuda.synchronize()
+        out.append(C.cpu().numpy().view(np.uint16))
+    assert np.array_equal(out[0], out[1])
+    assert oracle.compare(out[0], oracle_ref(oracle, A, B, N))[0] <= TOL_F16
+    with pytest.raises(smat.SmatError, match="row-major"):
+        C = torch.zeros((M, N), dtype=torch.int16, device=cuda)
+        smat.spmm(vals, rp, ci, to_dev(torch, B_rm, cuda), C, M, N, K, nnzb, plan=p, kernel=1, b_row_major=True)
+    p.close()

