@@ -6,7 +6,8 @@
 // and adds: -reorder (row + column clustering before blocking), -tau,
 //   -random_b (seeded uniform[-1,1] B instead of all ones), -use_plan, -kernel,
 //   -gpu_blocking (CSR -> BCSR on the device).  -filename also takes a binary container
-//   written by smat_convert.  Load, reorder and blocking times are logged apart from the SpMM time.
+//   written by smat_convert.  -lineplot [-lineplot_from=14 -lineplot_to=126 -lineplot_step=1] sweeps
+//   N = 8*mult like createLinePlot (common/tester.h:211-267) and appends "N, ms" lines to results_smat.csv.  Load, reorder and blocking times are logged apart from the SpMM time.
 #include <thread>
 
 #include "flags.h"
@@ -34,11 +35,20 @@ int main(int argc, char **argv)
          f.num("warmup_iterations", 1), f.num("profiling_iterations", 10), f.num("sleep_duration", 100),
          (int)f.flag("enable_check", false));
 
+    const bool lineplot = f.flag("lineplot", false);
+    const int lp_from = (int)f.num("lineplot_from", 14), lp_to = (int)f.num("lineplot_to", 126),
+              lp_step = (int)f.num("lineplot_step", 1);
+    if (lineplot && (lp_from < 1 || lp_to <= lp_from || lp_step < 1)) { HLOG("bad -lineplot_from/_to/_step"); return 2; }
+    // with -lineplot the plan is made for the widest N of the sweep
     Tester tester((size_t)f.num("warmup_iterations", 1), (size_t)f.num("profiling_iterations", 10),
-                  (size_t)f.num("sleep_duration", 100), f.flag("enable_check", false), n_mult, file,
+                  (size_t)f.num("sleep_duration", 100), f.flag("enable_check", false),
+                  lineplot ? lp_from + (lp_to - 1 - lp_from) / lp_step * lp_step : n_mult, file,
                   f.flag("reorder", false), (float)f.real("tau", 0.5), f.flag("random_b", false),
                   f.flag("use_plan", true), (int)f.num("kernel", SMAT_KERNEL_AUTO), f.flag("gpu_blocking", false));
-    if (f.flag("use_plan", true))
+    if (lineplot) {
+        if (!f.flag("use_plan", true)) { HLOG("-lineplot needs the plan (-use_plan)"); return 2; }
+        tester.createLinePlot("Smat-Plan-Kernel", lp_from, lp_to, lp_step);
+    } else if (f.flag("use_plan", true))
         tester.evaluatePlanned("Smat-Plan-Kernel");
     else
         tester.evaluateSparse2(mmaCBTKernel, "Mma-CBT-Kernel"); // the drop-in symbol, as in main.cu:99

@@ -85,6 +85,45 @@ public:
         evaluateSparse2(f, name);
     }
 
+    // N sweep of the reference harness (createLinePlot, common/tester.h:211-267): for
+    // N = 8*mult, mult in [from, to), time the kernel and append "N, ms" to results_smat.csv.
+    // The plan (built for the largest N of the sweep) is reused; B and C are re-made per N.
+    void createLinePlot(const std::string &name, int from, int to, int step)
+    {
+        HLOG("----------------- Sparse Lineplot %s -----------------", name.c_str());
+        double base_ms = 0, base_tflops = 0;
+        for (int mult = from; mult < to; mult += step) {
+            const size_t N = (size_t)mult * 8;
+            delete B_; delete C_;
+            B_ = new Matrix(A_->getCol(), N, "Matrix B for sparse", true, 0xB);
+            C_ = new Matrix(A_->getRow(), N, "Matrix C for sparse");
+            C_->memSetHost(); C_->moveToDevice();
+            auto f = [this](half *v, int *rp, int *ci, half *B, half *C, size_t M, size_t n, size_t K, size_t nnzb,
+                            int *, int *) {
+                smat_spmm_opts o = {SMAT_B_COL_MAJOR, SMAT_C_F16, kernel_, 0, nullptr};
+                SMAT_CHECK(smat_spmm_bcsr_f16_ex(v, rp, ci, B, C, M, n, K, nnzb, &o, plan_));
+            };
+            for (size_t i = 0; i < warmup_; ++i) call(f);
+            void *e0, *e1;
+            SMAT_CHECK(smat_event_create(&e0));
+            SMAT_CHECK(smat_event_create(&e1));
+            SMAT_CHECK(smat_event_record(e0, nullptr));
+            for (size_t i = 0; i < iters_; ++i) call(f);
+            SMAT_CHECK(smat_event_record(e1, nullptr));
+            SMAT_CHECK(smat_device_synchronize());
+            float ev = 0;
+            SMAT_CHECK(smat_event_elapsed_ms(e0, e1, &ev));
+            smat_event_destroy(e0); smat_event_destroy(e1);
+            const double ms = ev / (double)iters_;
+            const double tflops = (double)A_->getNonzeroblocks() * 256.0 * 2.0 * (double)N * 1e-12 / (ms * 1e-3);
+            if (base_ms == 0) { base_ms = ms; base_tflops = tflops; }
+            FILE *fout = fopen("results_smat.csv", "a");
+            if (fout) { fprintf(fout, "%zu, %lf\n", N, ms); fclose(fout); }
+            HLOG("%s exit, N = %zu, profiling time: %.4f ms (%.2f%%), throughput: %.3f TFLOPS (%.2f%%)", name.c_str(), N,
+                 ms, ms / base_ms * 100, tflops, tflops / base_tflops * 100);
+        }
+    }
+
     double lastMs() const { return event_ms_; }
 
 private:

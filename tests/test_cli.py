@@ -93,3 +93,18 @@ def test_hgemm_reads_binary_container(tmp_path):
     blocks = [ln.split("]")[-1] for ln in run.stderr.splitlines() if "nonzero blocks," in ln]
     blocks2 = [ln.split("]")[-1] for ln in run2.stderr.splitlines() if "nonzero blocks," in ln]
     assert blocks and blocks == blocks2
+
+
+@pytest.mark.gpu
+def test_hgemm_lineplot_sweeps_n(tmp_path):
+    """createLinePlot of the reference harness (common/tester.h:211-267): one "N, ms" line per N = 8*mult."""
+    d = gen.stencil27(10)
+    mtx = tmp_path / "stencil10.mtx"
+    write_mtx(mtx, d)
+    cmd = [os.path.join(BIN, "hgemm"), f"-filename={mtx}", "-random_b", "-warmup_iterations=1", "-profiling_iterations=2",
+           "-sleep_duration=1", "-lineplot", "-lineplot_from=14", "-lineplot_to=30", "-lineplot_step=5"]
+    run = subprocess.run(cmd, cwd=tmp_path, capture_output=True, text=True, timeout=120)
+    assert run.returncode == 0, run.stderr[-2000:]
+    lines = (tmp_path / "results_smat.csv").read_text().strip().splitlines()
+    assert [int(ln.split(",")[0]) for ln in lines] == [112, 152, 192, 232]
+    assert all(float(ln.split(",")[1]) > 0 for ln in lines)

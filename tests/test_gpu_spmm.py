@@ -396,3 +396,31 @@ def test_compact_kernel_row_major_b(smat, cuda, oracle):
         C = torch.zeros((M, N), dtype=torch.int16, device=cuda)
         smat.spmm(vals, rp, ci, to_dev(torch, B_rm, cuda), C, M, N, K, nnzb, plan=p, kernel=1, b_row_major=True)
     p.close()
+
+
+def test_compact_kernel_config2_full_size(smat, cuda, oracle):
+    """Config 2 at its real size (16384 x 16384, 0.1 %, N = 256), whole result against the oracle."""
+    d = gen.erdos_renyi(16384, 0.001)
+    A = bcsr_of(smat, d)
+    N = 256
+    B = gen.dense_b(A["K"], N, seed=0xB0000002, dist="normal")
+    C, info = gpu_spmm_compact(smat, cuda, A, B, N, kernel=0)
+    assert info["kernel"] == COMPACT and info["compact_cols"] <= int(d["row_ptr"][-1])
+    assert oracle.compare(C, oracle_ref(oracle, A, B, N))[0] <= TOL_F16
+
+
+def test_compact_kernel_power_law_rows(smat, cuda, oracle):
+    """R-MAT scale 15: block rows of very different length, the longest split into chunks."""
+    d = gen.rmat(15, 16, seed=21)
+    A = bcsr_of(smat, d)
+    N = 128
+    B = gen.dense_b(A["K"], N, seed=9, dist="uniform")
+    C, info = gpu_spmm_compact(smat, cuda, A, B, N, kernel=0)
+    assert info["kernel"] == COMPACT
+    assert oracle.compare(C, oracle_ref(oracle, A, B, N))[0] <= TOL_F16
+    # linearity in B, a size-independent property: A (2 B) = 2 (A B) bit for bit in the fp32 output
+    # (scaling by two is exact in every product and every partial sum)
+    B2 = (B.view(np.float16) * np.float16(2)).view(np.uint16)
+    C32, _ = gpu_spmm_compact(smat, cuda, A, B, N, kernel=0, c_f32=True)
+    C32_2, _ = gpu_spmm_compact(smat, cuda, A, B2, N, kernel=0, c_f32=True)
+    assert np.array_equal(C32 * np.float32(2), C32_2)
