@@ -39,6 +39,7 @@ MEASURED_TRAFFIC = {
 
 
 INFO = {}  # facts about the generated workload that go into the config of the result line
+PERM_FILE = None
 
 
 def build_workload(name):
@@ -77,9 +78,20 @@ def build_workload(name):
             b = smat_amd.csr_to_bcsr(d["M"], d["K"], rp, ci, v)
         A = {"M": b.M, "K": b.K, "b_row_ptr": b.row_ptr, "b_col_idx": b.col_idx, "b_val": b.val, "nnzb": b.nnzb}
         N, bdist, bseed = 256, "normal", 0xB0000002
-    elif name == "rmat_s20_deg16_N128":
+    elif name in ("rmat_s20_deg16_N128", "rmat_s20_deg16_reordered_N128"):
         d = gen.rmat(20, 16)
         b = smat_amd.csr_to_bcsr(d["M"], d["K"], d["row_ptr"], d["col_idx"], d["val"])
+        if "reordered" in name:
+            # the reorder of 2^20 rows takes most of an hour on the host: its permutations come from a
+            # file (npz with perm_rows, perm_cols, reorder_s) written by an earlier smat_amd.reorder_csr run
+            if not PERM_FILE:
+                raise SystemExit("rmat_s20_deg16_reordered_N128 needs --perm-file")
+            z = np.load(PERM_FILE)
+            INFO["reorder_s"] = float(z["reorder_s"])
+            INFO["nnzb_before_reorder"] = int(b.nnzb)
+            rp, ci, v = smat_amd.permute_csr(d["M"], d["K"], d["row_ptr"], d["col_idx"], d["val"],
+                                             z["perm_rows"], z["perm_cols"])
+            b = smat_amd.csr_to_bcsr(d["M"], d["K"], rp, ci, v)
         A = {"M": b.M, "K": b.K, "b_row_ptr": b.row_ptr, "b_col_idx": b.col_idx, "b_val": b.val, "nnzb": b.nnzb}
         N, bdist, bseed = 128, "uniform", 0xB0000003
     else:
@@ -178,6 +190,7 @@ def main():
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--no-attach-values", action="store_true",
                     help="do not let the plan look at the block values (the compact kernel, id 5, needs them)")
+    ap.add_argument("--perm-file", default=None, help="npz with perm_rows / perm_cols / reorder_s (reordered R-MAT workload)")
     ap.add_argument("--calibration-copy-mib", type=int, default=0,
                     help="also run one plain device copy of this many MiB (a kernel of known HBM traffic, "
                          "to scale rocprofv3 FETCH_SIZE / WRITE_SIZE readings)")
@@ -191,6 +204,8 @@ def main():
 
     assert torch.cuda.is_available(), "bench.py needs a GPU"
     dev = torch.device("cuda:0")
+    global PERM_FILE
+    PERM_FILE = args.perm_file
     A, B, N = build_workload(args.workload)
     M, K, nnzb = A["M"], A["K"], A["nnzb"]
 
