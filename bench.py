@@ -31,6 +31,8 @@ PEAK_HBM_GBS = 8000.0      # MI355X HBM3E
 # device copy of known size (summaries under profiles/): (workload, kernel id) -> bytes
 MEASURED_TRAFFIC = {
     ("block_pruned_8192_10pct_N4096", 2): 143442 * 1024 * 2.0 + 65824 * 1024 * 1.0,
+    # row-wise kernel + repack kernel
+    ("block_pruned_8192_10pct_N4096", 1): (247966 + 32783) * 1024 * 2.0 + (65538 + 65536) * 1024 * 1.0,
     # compact kernel + transpose kernel (+ reduce kernel for the split rows of R-MAT)
     ("er_16384_0.1pct_reordered_N256", 5): (25992 + 4111) * 1024 * 2.0 + (8192 + 8192) * 1024 * 1.0,
     ("rmat_s20_deg16_N128", 5): (1531955 + 131089 + 37914) * 1024 * 2.0 + (327815 + 262144 + 10068) * 1024 * 1.0,

@@ -233,11 +233,12 @@ extern "C" int smat_plan_create(smat_plan **out, const int32_t *row_ptr_host,
     }
     // The sweep kernel pays one pass over the B panel per group of 32 block rows,
     // whatever the sparsity, and shares each staged slab between the blocks of the group
-    // that sit in that block column: it overtakes the row-wise kernel at about 10% of the
-    // blocks present, with N wide enough for many panels.
+    // that sit in that block column.  At 10% of the blocks present (8192 x 8192, N = 4096) it
+    // takes 180 us against 176 us for the row-wise kernel on repacked B; its share of reused
+    // slabs grows with the density, the row-wise kernel's work does not shrink: taken from 12%.
     bool sweep = want == SMAT_KERNEL_SWEEP;
     if (want == SMAT_KERNEL_AUTO && col_idx_host && n_hint >= 512 && mb >= 2 * (size_t)SWEEP_G &&
-        (double)nnzb >= 0.08 * (double)mb * (double)kb)
+        (double)nnzb >= 0.12 * (double)mb * (double)kb)
         sweep = true;
     if (sweep && nnzb >= (size_t)1 << 23) { // the sweep kernel addresses blocks with 32-bit byte offsets
         if (want == SMAT_KERNEL_SWEEP) {

@@ -31,7 +31,7 @@ struct SpmmArgs {
     void *C;
     size_t M, N, K, nnzb;
     bool c_f32;
-    int panel_tiles;       // 0 = choose from N; else 1, 2, 4 or 8 n-tiles of 16 per wavefront
+    int panel_tiles;       // 0 = choose from N; else 1, 2, 4, 8 or 16 n-tiles of 16 per wavefront
     const WorkItem *items; // device; nullptr = one item per block row
     int n_items;
     const SplitRow *split_rows; // device

@@ -299,7 +299,8 @@ static hipError_t launch_rowwise_tn(const SpmmArgs &a, hipStream_t st)
 
 int rowwise_panel_tiles(size_t N, int requested, size_t n_items)
 {
-    if (requested == 1 || requested == 2 || requested == 4 || requested == 8) return requested;
+    if (requested == 1 || requested == 2 || requested == 4 || requested == 8 || requested == 16) return requested;
+    if (N >= 1024) return 16; // 256 columns per wavefront: every A block is read once per 256 columns of C
     if (N >= 512) return 8;
     // Below that, 64-column panels: measured faster than 128-column ones even where the work
     // list alone fills the chip (R-MAT scale 20, N = 128: 13.8 ms against 18.2 ms), more
@@ -320,6 +321,7 @@ hipError_t launch_rowwise(const SpmmArgs &a, hipStream_t st)
         if (e != hipSuccess) return e;
     }
     switch (rowwise_panel_tiles(a.N, a.panel_tiles, (size_t)a.n_items)) {
+    case 16: e = launch_rowwise_tn<16>(a, st); break;
     case 8: e = launch_rowwise_tn<8>(a, st); break;
     case 4: e = launch_rowwise_tn<4>(a, st); break;
     case 2: e = launch_rowwise_tn<2>(a, st); break;
