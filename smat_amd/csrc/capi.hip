@@ -348,8 +348,9 @@ extern "C" int smat_plan_attach_values(smat_plan *p, const uint16_t *vals, const
     // (9.6 per block), unless a kernel was asked for.
     const bool take = p->kernel_requested == SMAT_KERNEL_COMPACT ||
                       (p->kernel_requested == SMAT_KERNEL_AUTO && (double)c->n_cols < 0.6 * 16.0 * (double)p->nnzb);
-    if (!take) { // nothing will use the list: the plan stays as it was
+    if (!take) { // nothing will use the list: the plan keeps (or goes back to) a dense kernel
         compact_destroy(c);
+        if (p->kernel == SMAT_KERNEL_COMPACT) p->kernel = p->d_ops ? SMAT_KERNEL_SWEEP : SMAT_KERNEL_ROWWISE;
         return SMAT_OK;
     }
     if (!p->d_bt) e = hipMalloc(&p->d_bt, p->K * p->n_cap * sizeof(uint16_t));
