@@ -107,6 +107,11 @@ extern "C" int smat_spmm_bcsr_f16_ex(const uint16_t *vals, const int32_t *row_pt
     if (kernel != SMAT_KERNEL_ROWWISE && kernel != SMAT_KERNEL_SWEEP && kernel != SMAT_KERNEL_COMPACT)
         return set_error(SMAT_ERR_INVALID, "unknown kernel id %d", kernel);
     hipError_t e;
+    if (kernel == SMAT_KERNEL_SWEEP && K * N >= ((size_t)1 << 31)) { // its B copies use 32-bit byte offsets
+        if (o.kernel == SMAT_KERNEL_SWEEP)
+            return set_error(SMAT_ERR_UNSUPPORTED, "SMAT_KERNEL_SWEEP takes a B smaller than 4 GiB");
+        kernel = SMAT_KERNEL_ROWWISE;
+    }
     if (o.b_layout == SMAT_B_ROW_MAJOR && kernel != SMAT_KERNEL_COMPACT)
         return set_error(SMAT_ERR_UNSUPPORTED,
                          "row-major B (B[k*N+n]) is implemented for SMAT_KERNEL_COMPACT only; the other kernels "
@@ -234,11 +239,11 @@ extern "C" int smat_plan_create(smat_plan **out, const int32_t *row_ptr_host,
     // The sweep kernel pays one pass over the B panel per group of 32 block rows,
     // whatever the sparsity, and shares each staged slab between the blocks of the group
     // that sit in that block column.  At 10% of the blocks present (8192 x 8192, N = 4096) it
-    // takes 180 us against 176 us for the row-wise kernel on repacked B; its share of reused
-    // slabs grows with the density, the row-wise kernel's work does not shrink: taken from 12%.
+    // takes 160 us against 173 us for the row-wise kernel on repacked B; its share of reused
+    // slabs grows with the density, the row-wise kernel's work does not shrink: taken from 9.5%.
     bool sweep = want == SMAT_KERNEL_SWEEP;
     if (want == SMAT_KERNEL_AUTO && col_idx_host && n_hint >= 512 && mb >= 2 * (size_t)SWEEP_G &&
-        (double)nnzb >= 0.12 * (double)mb * (double)kb)
+        (double)nnzb >= 0.095 * (double)mb * (double)kb)
         sweep = true;
     if (sweep && nnzb >= (size_t)1 << 23) { // the sweep kernel addresses blocks with 32-bit byte offsets
         if (want == SMAT_KERNEL_SWEEP) {
@@ -251,7 +256,7 @@ extern "C" int smat_plan_create(smat_plan **out, const int32_t *row_ptr_host,
         const size_t n_rg = (mb + SWEEP_G - 1) / SWEEP_G;
         std::vector<int32_t> rg_ptr(n_rg + 1, 0), chunk_ids;
         std::vector<SweepOp> ops; // records * SWEEP_WAVES * SWEEP_CAP table slots
-        const SweepOp empty_slot = {-1, -1, 0, 0};
+        const SweepOp empty_slot = {SWEEP_EMPTY_SLOT, SWEEP_EMPTY_SLOT};
         struct Ent { int32_t chunk, wave, r, slab, p; };
         std::vector<Ent> ents;
         constexpr int CAPR = SWEEP_CAP / SWEEP_RW; // table slots per block row
@@ -285,12 +290,10 @@ extern "C" int smat_plan_create(smat_plan **out, const int32_t *row_ptr_host,
                             const bool pair = i + 1 < ents.size() && ents[i + 1].chunk == chunk &&
                                               ents[i + 1].wave == w && ents[i + 1].r == r;
                             SweepOp op;
-                            op.p1 = ents[i].p;
-                            op.p2 = pair ? ents[i + 1].p : -1;
+                            op.w0 = (uint32_t)ents[i].p | ((uint32_t)ents[i].slab << 24);
                             // a single block: the upper MFMA half gets zeros of A and reads the same slab
-                            auto lds_off = [](int32_t slab) { return (slab / 8) * (16 * SWEEP_TN * 256) + (slab % 8) * 32; };
-                            op.meta = lds_off(ents[i].slab) | (lds_off(pair ? ents[i + 1].slab : ents[i].slab) << 16);
-                            op.pad = 0;
+                            op.w1 = pair ? ((uint32_t)ents[i + 1].p | ((uint32_t)ents[i + 1].slab << 24))
+                                         : (SWEEP_NO_BLOCK | ((uint32_t)ents[i].slab << 24));
                             list.push_back(op);
                             i += pair ? 2 : 1;
                         }
@@ -324,6 +327,10 @@ extern "C" int smat_plan_create(smat_plan **out, const int32_t *row_ptr_host,
         upload((void **)&p->d_rg_chunk_ptr, rg_ptr.data(), rg_ptr.size() * sizeof(int32_t));
         upload((void **)&p->d_chunk_ids, chunk_ids.data(), chunk_ids.size() * sizeof(int32_t));
         upload((void **)&p->d_ops, ops.data(), ops.size() * sizeof(SweepOp));
+        if (p->d_bpack && want == SMAT_KERNEL_AUTO) { // the sweep kernel reads B in place
+            (void)hipFree(p->d_bpack);
+            p->d_bpack = nullptr;
+        }
     }
     if (e != hipSuccess) {
         smat_plan_destroy(p);

@@ -41,17 +41,18 @@ struct SpmmArgs {
 };
 
 // One MFMA worth of work in the sweep kernel: two blocks of the same block row
-// whose block columns lie in the same K chunk (p2 < 0: a single block; p1 < 0: an
-// empty table slot).  meta = LDS byte offset of p1's slab | that of p2's slab << 16,
-// offset = (slab / 8) * 128 * 256 + (slab % 8) * 32 with slab = block column
-// relative to the first block column of the chunk (a single repeats p1's slab).
+// whose block columns lie in the same K chunk.  w0 = index of the first block |
+// its slab << 24, w1 = the same for the second block; slab = block column relative
+// to the first block column of the chunk.  A single block has SWEEP_NO_BLOCK in
+// the low 24 bits of w1 (and repeats the slab); an empty table slot has w0 = ~0.
 // Table slot k of a (record, wavefront) serves local block row k / (SWEEP_CAP / SWEEP_RW).
+// The 64 bytes of a (record, wavefront) table are read with one scalar load.
 struct SweepOp {
-    int32_t p1;
-    int32_t p2;
-    int32_t meta;
-    int32_t pad;
+    uint32_t w0;
+    uint32_t w1;
 };
+constexpr uint32_t SWEEP_NO_BLOCK = 0xFFFFFFu;
+constexpr uint32_t SWEEP_EMPTY_SLOT = 0xFFFFFFFFu;
 
 // Geometry of the sweep kernel (fixed at compile time).
 constexpr int SWEEP_TN = 8;     // n-tiles of 16 per workgroup panel -> 128 columns

@@ -31,6 +31,7 @@
 #include <hip/hip_runtime.h>
 #include <stdint.h>
 
+#include <type_traits>
 #include "spmm_kernels.h"
 
 namespace smat {
@@ -66,39 +67,51 @@ __device__ __forceinline__ void fill_issue(unsigned char *stage, const uint16_t 
     const int q = lane >> 4, ps = lane & 15;
     // swizzle_of_n(n) = q | bit4(n) << 2 | bit5(n) << 3 with bit4(n) = wave/4, bit5(n) = it & 1
     const int ls0 = ps ^ (q | (((wave >> 2) & 1) << 2));
-    const long kmax = K - 8;
+    // Source address = wave-uniform base (column block of the instruction) + 32-bit lane
+    // offset: the launcher checks that B is smaller than 4 GiB.
+    const uint32_t kmax = (uint32_t)K - 8u;
+    const uint32_t col_off = (uint32_t)(n0 + wave * 4 + q) * (uint32_t)K; // in elements
+    const uint32_t k0 = (uint32_t)chunk * (S * 16);
 #pragma unroll
     for (int it = 0; it < FILL_ITERS; it++) {
         const int nrow = n0 + (it & 3) * 32 + wave * 4; // first of 4 columns, wave-uniform
         if (nrow >= N) continue;                          // N % 8 == 0: all four or none
-        const int ls = ls0 ^ ((it & 1) << 3);
-        long k = (long)chunk * (S * 16) + (it >> 2) * 128 + ls * 8;
+        const uint32_t ls = (uint32_t)(ls0 ^ ((it & 1) << 3));
+        uint32_t k = k0 + (it >> 2) * 128 + ls * 8;
         k = k < kmax ? k : kmax; // slabs past K are never referenced; keep the read in bounds
-        const uint16_t *src = B + (long)(nrow + q) * K + k;
+        const uint32_t voff = (col_off + k) * 2u;
+        const uint16_t *sbase = B + (long)((it & 3) * 32) * K;
         // Issued from inline assembly on purpose: the compiler orders every later LDS
         // read after a global->LDS copy it knows about (it cannot tell the two stages
         // apart) and would wait for the copy before the MFMA work of the current
         // chunk.  The copies are waited for explicitly (vmcnt(0)) before the barrier.
         const uint32_t dst = (uint32_t)(uintptr_t)(__attribute__((address_space(3))) void *)(
             stage + (size_t)(it * W + wave) * 1024);
-        asm volatile("s_mov_b32 m0, %1\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, off"
+        asm volatile("s_mov_b32 m0, %2\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, %1"
                      :
-                     : "v"(src), "s"(dst)
+                     : "v"(voff), "s"(sbase), "s"(dst)
                      : "memory", "m0");
     }
 }
 
 } // namespace
 
-typedef int i32x4 __attribute__((ext_vector_type(4)));
+typedef uint32_t u32x16 __attribute__((ext_vector_type(16)));
 
-// Lane l of the returned vector holds slot l % CAP of the op table of (record,
-// wavefront).  Every lane loads (no branch): a load inside a branch cannot be
-// counted by the compiler's vmcnt bookkeeping and would force full waits later.
-__device__ __forceinline__ i32x4 load_op_table(const SweepOp *__restrict__ ops, int record, int wave, int lane)
+// The op table of (record, wavefront): 8 slots of {w0, w1}.  Read through the constant
+// address space with a wave-uniform address: one scalar load, no vector memory
+// instruction and no v_readlane to get at a slot.
+__device__ __forceinline__ u32x16 load_op_table(const SweepOp *__restrict__ ops, int record, int wave)
 {
-    return *reinterpret_cast<const i32x4 *>(ops + ((long)record * W + wave) * SWEEP_CAP +
-                                            (lane & (SWEEP_CAP - 1)));
+    static_assert(SWEEP_CAP * sizeof(SweepOp) == sizeof(u32x16), "one table = 16 dwords");
+    typedef const __attribute__((address_space(4))) u32x16 *table_ptr;
+    return *(table_ptr)(uintptr_t)(ops + ((long)record * W + wave) * SWEEP_CAP);
+}
+
+// LDS byte offset (without the per-lane XOR) of a slab of the staged chunk
+__device__ __forceinline__ uint32_t slab_offset(uint32_t slab)
+{
+    return (slab >> 3) * (uint32_t)(NT * 256) + (slab & 7u) * 32u;
 }
 
 template <bool C_F32>
@@ -139,26 +152,28 @@ __global__ __launch_bounds__(THREADS) void spmm_sweep_kernel(
     const int c_begin = rg_chunk_ptr[rg], c_end = rg_chunk_ptr[rg + 1];
     const uint32_t a_lane_bytes = (uint32_t)(i16 * 16 + kh * 8) * 2u; // this lane's 16 bytes inside a block
     const f16x8 zero8 = {0, 0, 0, 0, 0, 0, 0, 0};
-    const i32x4 empty_table = {-1, -1, 0, 0};
 
-    // A operands of one chunk: slot k <- the two blocks of op k (lanes 0-31: p1, 32-63: p2).
-    // Loads are unconditional: an empty slot or the missing second block of a single
-    // re-reads a valid block (its data is never used, or is zeroed at use).
-    auto load_a = [&](f16x8 (&dst)[CAP], const i32x4 &tab) {
+    // A operands of one chunk: slot k <- the two blocks of op k (lanes 0-31: first block,
+    // 32-63: second).  Empty slots load nothing: a vector memory instruction costs the
+    // load path of the CU 16 clocks whatever it fetches.  The missing second block of a
+    // single re-reads the first (zeroed at use).
+    auto load_a = [&](f16x8 (&dst)[CAP], const u32x16 &tab) {
 #pragma unroll
         for (int k = 0; k < CAP; k++) {
-            const int p1 = __builtin_amdgcn_readlane(tab[0], k);
-            const int p2 = __builtin_amdgcn_readlane(tab[1], k);
-            // empty slot: every lane reads the first 16 bytes of vals (one cache line)
-            const uint32_t b1 = p1 < 0 ? 0u : (uint32_t)p1 * 512u;
-            const uint32_t b2 = p2 < 0 ? b1 : (uint32_t)p2 * 512u;
-            const uint32_t lo = p1 < 0 ? 0u : a_lane_bytes;
-            const uint32_t off = (sel ? b2 : b1) + lo; // nnzb * 512 < 2^32 is checked by the plan
-            dst[k] = *reinterpret_cast<const f16x8 *>(reinterpret_cast<const char *>(vals) + off);
+            const uint32_t w0 = tab[2 * k], w1 = tab[2 * k + 1];
+            if (w0 != SWEEP_EMPTY_SLOT) {
+                const uint32_t b1 = (w0 & 0xFFFFFFu) * 512u; // nnzb < 2^23 is checked by the plan
+                const uint32_t p2 = w1 & 0xFFFFFFu;
+                const uint32_t b2 = p2 == SWEEP_NO_BLOCK ? b1 : p2 * 512u;
+                const uint32_t off = (sel ? b2 : b1) + a_lane_bytes;
+                dst[k] = *reinterpret_cast<const f16x8 *>(reinterpret_cast<const char *>(vals) + off);
+            }
         }
     };
 
-    i32x4 tab_cur = empty_table, tab_nxt = empty_table, tab_nx2 = empty_table;
+    u32x16 tab_cur, tab_nxt, tab_nx2;
+#pragma unroll
+    for (int k = 0; k < 16; k++) { tab_cur[k] = SWEEP_EMPTY_SLOT; tab_nxt[k] = SWEEP_EMPTY_SLOT; tab_nx2[k] = SWEEP_EMPTY_SLOT; }
 
     f16x8 a_cur[CAP], a_nxt[CAP];
 #pragma unroll
@@ -167,8 +182,8 @@ __global__ __launch_bounds__(THREADS) void spmm_sweep_kernel(
     int stage = 0;
     if (c_begin < c_end) {
         const int last = c_end - 1;
-        tab_cur = load_op_table(ops, c_begin, wave, lane);
-        tab_nxt = load_op_table(ops, c_begin + 1 < last ? c_begin + 1 : last, wave, lane);
+        tab_cur = load_op_table(ops, c_begin, wave);
+        tab_nxt = load_op_table(ops, c_begin + 1 < last ? c_begin + 1 : last, wave);
         fill_issue(lds, B, chunk_ids[c_begin] & ~SWEEP_CONT_FLAG, n0, N, K, wave, lane);
         load_a(a_cur, tab_cur);
     }
@@ -176,62 +191,62 @@ __global__ __launch_bounds__(THREADS) void spmm_sweep_kernel(
     __syncthreads();
 
     for (int ci = c_begin; ci < c_end; ci++) {
-        // ---- issue everything chunk ci+1 (and the table of ci+2) needs ----
-        // Past the end the last record is simply loaded again: no branches around loads.
         const int last = c_end - 1;
-        tab_nx2 = load_op_table(ops, ci + 2 < last ? ci + 2 : last, wave, lane);
-        load_a(a_nxt, tab_nxt);
-        // A record that continues the chunk of the previous record (its ops did not
-        // fit one table) has bit 30 set: no B copy, the LDS stage stays.
-        int next_chunk = 0;
         bool next_is_new = false;
-        if (ci + 1 < c_end) {
-            next_chunk = chunk_ids[ci + 1];
-            next_is_new = !(next_chunk & SWEEP_CONT_FLAG);
-            if (next_is_new)
-                fill_issue(lds + (stage ^ 1) * STAGE_BYTES, B, next_chunk, n0, N, K, wave, lane);
-        }
-
-        // ---- MFMA work of chunk ci: registers and LDS only ----
-        const unsigned char *cur = lds + stage * STAGE_BYTES + rd_base;
-#pragma unroll
-        for (int k = 0; k < CAP; k++) {
-            // slot k belongs to block row k / CAPR of this wavefront: the accumulator
-            // registers of every slot are fixed at compile time
-            constexpr int CAPR = CAP / RW;
-            const int p1 = __builtin_amdgcn_readlane(tab_cur[0], k);
-            if (p1 >= 0) {
-                // meta = LDS byte offset of the slab of p1 | that of p2 << 16 (without the
-                // per-lane XOR): slab group * NT * 256 + (slab % 8) * 32
-                const uint32_t meta = (uint32_t)__builtin_amdgcn_readlane(tab_cur[2], k);
-                const uint32_t soff = sel ? (meta >> 16) : (meta & 0xffffu);
-                const unsigned char *bp = cur + (soff ^ lane_xor);
-                f16x8 av = a_cur[k];
-                if (__builtin_amdgcn_readlane(tab_cur[1], k) < 0) // single: no second block
-                    av = sel ? zero8 : av;
-#pragma unroll
-                for (int u = 0; u < TN / 4; u++) {
-                    f16x8 b[4];
-#pragma unroll
-                    for (int tt = 0; tt < 4; tt++)
-                        b[tt] = *reinterpret_cast<const f16x8 *>(bp + (64 * u + 4 * tt) * ROW_BYTES);
-#pragma unroll
-                    for (int tt = 0; tt < 4; tt++)
-                        acc[k / CAPR][u * 4 + tt] = __builtin_amdgcn_mfma_f32_16x16x32_f16(
-                            b[tt], av, acc[k / CAPR][u * 4 + tt], 0, 0, 0);
-                }
-                // order of the 8 LDS reads and 8 MFMAs of this op: four reads ahead, then one
-                // MFMA per further read, so an MFMA never waits on the read issued just before it
-                __builtin_amdgcn_sched_group_barrier(0x100, 4, 0);
-#pragma unroll
-                for (int q = 0; q < 4; q++) {
-                    __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
-                    __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);
-                }
-                __builtin_amdgcn_sched_group_barrier(0x008, 4, 0);
+        // ---- everything chunk ci+1 (and the table of ci+2) needs ----
+        // Past the end the last record's table is simply loaded again.
+        auto do_loads = [&]() {
+            tab_nx2 = load_op_table(ops, ci + 2 < last ? ci + 2 : last, wave);
+            if (ci + 1 < c_end) {
+                load_a(a_nxt, tab_nxt);
+                // A record that continues the chunk of the previous record (its ops did not
+                // fit one table) has bit 30 set: no B copy, the LDS stage stays.
+                const int next_chunk = chunk_ids[ci + 1];
+                next_is_new = !(next_chunk & SWEEP_CONT_FLAG);
+                if (next_is_new)
+                    fill_issue(lds + (stage ^ 1) * STAGE_BYTES, B, next_chunk, n0, N, K, wave, lane);
             }
-        }
-
+        };
+        // ---- MFMA work of chunk ci: registers and LDS only ----
+        auto do_compute = [&](auto k_begin, auto k_end) {
+            const unsigned char *cur = lds + stage * STAGE_BYTES + rd_base;
+#pragma unroll
+            for (int k = decltype(k_begin)::value; k < decltype(k_end)::value; k++) {
+                // slot k belongs to block row k / CAPR of this wavefront: the accumulator
+                // registers of every slot are fixed at compile time
+                constexpr int CAPR = CAP / RW;
+                const uint32_t w0 = tab_cur[2 * k], w1 = tab_cur[2 * k + 1];
+                if (w0 != SWEEP_EMPTY_SLOT) {
+                    const uint32_t soff = sel ? slab_offset(w1 >> 24) : slab_offset(w0 >> 24);
+                    const unsigned char *bp = cur + (soff ^ lane_xor);
+                    f16x8 av = a_cur[k];
+                    if ((w1 & 0xFFFFFFu) == SWEEP_NO_BLOCK) // single: no second block
+                        av = sel ? zero8 : av;
+#pragma unroll
+                    for (int u = 0; u < TN / 4; u++) {
+                        f16x8 b[4];
+#pragma unroll
+                        for (int tt = 0; tt < 4; tt++)
+                            b[tt] = *reinterpret_cast<const f16x8 *>(bp + (64 * u + 4 * tt) * ROW_BYTES);
+#pragma unroll
+                        for (int tt = 0; tt < 4; tt++)
+                            acc[k / CAPR][u * 4 + tt] = __builtin_amdgcn_mfma_f32_16x16x32_f16(
+                                b[tt], av, acc[k / CAPR][u * 4 + tt], 0, 0, 0);
+                    }
+                    // order of the 8 LDS reads and 8 MFMAs of this op: four reads ahead, then one
+                    // MFMA per further read, so an MFMA never waits on the read issued just before it
+                    __builtin_amdgcn_sched_group_barrier(0x100, 4, 0);
+#pragma unroll
+                    for (int q = 0; q < 4; q++) {
+                        __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
+                        __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);
+                    }
+                    __builtin_amdgcn_sched_group_barrier(0x008, 4, 0);
+                }
+            }
+        };
+        do_loads();
+        do_compute(std::integral_constant<int, 0>(), std::integral_constant<int, CAP>());
         __builtin_amdgcn_s_waitcnt(0x0f70); // vmcnt(0): next chunk's B, A and table have landed
         __syncthreads();
         if (next_is_new) stage ^= 1;
@@ -301,3 +316,4 @@ hipError_t launch_sweep(const SweepArgs &a, hipStream_t st)
 }
 
 } // namespace smat
+
