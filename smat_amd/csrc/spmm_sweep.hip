@@ -25,13 +25,17 @@
 //    the B panel of chunk c+1 (global -> LDS asynchronously with
 //    global_load_lds_dwordx4, no staging registers, into the other LDS stage).
 //    The MFMA loop itself touches only registers and LDS.  One barrier per chunk.
+//  * Vector memory instructions are the scarce resource of the load phase: the load
+//    path of a CU takes about one 64-lane instruction (up to 1 KiB) per 16 clocks and
+//    the issuing wavefront stalls meanwhile.  So the op tables are read with scalar
+//    loads (64 bytes per record and wavefront), empty table slots load no A, and the
+//    B copies move 16 bytes per lane from a scalar base plus a 32-bit lane offset.
 //
 // Same operand semantics as the reference launcher
 // (src/cuda_hgemm/src/mma/mmaCBT.cu:83-88).
 #include <hip/hip_runtime.h>
 #include <stdint.h>
 
-#include <type_traits>
 #include "spmm_kernels.h"
 
 namespace smat {
@@ -208,10 +212,10 @@ __global__ __launch_bounds__(THREADS) void spmm_sweep_kernel(
             }
         };
         // ---- MFMA work of chunk ci: registers and LDS only ----
-        auto do_compute = [&](auto k_begin, auto k_end) {
+        auto do_compute = [&]() {
             const unsigned char *cur = lds + stage * STAGE_BYTES + rd_base;
 #pragma unroll
-            for (int k = decltype(k_begin)::value; k < decltype(k_end)::value; k++) {
+            for (int k = 0; k < CAP; k++) {
                 // slot k belongs to block row k / CAPR of this wavefront: the accumulator
                 // registers of every slot are fixed at compile time
                 constexpr int CAPR = CAP / RW;
@@ -246,7 +250,7 @@ __global__ __launch_bounds__(THREADS) void spmm_sweep_kernel(
             }
         };
         do_loads();
-        do_compute(std::integral_constant<int, 0>(), std::integral_constant<int, CAP>());
+        do_compute();
         __builtin_amdgcn_s_waitcnt(0x0f70); // vmcnt(0): next chunk's B, A and table have landed
         __syncthreads();
         if (next_is_new) stage ^= 1;
