@@ -65,6 +65,14 @@ static int check_shapes(const void *vals, const void *row_ptr, const void *col_i
     return SMAT_OK;
 }
 
+// The sweep kernel runs one workgroup per (group of SWEEP_G block rows, panel of 128 columns),
+// one workgroup per CU at a time.
+static bool sweep_fills_device(size_t mb, size_t n)
+{
+    const size_t n_rg = (mb + SWEEP_G - 1) / SWEEP_G, n_panels = (n + 16 * SWEEP_TN - 1) / (16 * SWEEP_TN);
+    return n_rg * n_panels >= 256;
+}
+
 extern "C" int smat_spmm_bcsr_f16_ex(const uint16_t *vals, const int32_t *row_ptr,
                                       const int32_t *col_idx, const uint16_t *B, void *C, size_t M,
                                       size_t N, size_t K, size_t nnzb, const smat_spmm_opts *opts,
@@ -112,6 +120,9 @@ extern "C" int smat_spmm_bcsr_f16_ex(const uint16_t *vals, const int32_t *row_pt
             return set_error(SMAT_ERR_UNSUPPORTED, "SMAT_KERNEL_SWEEP takes a B smaller than 4 GiB");
         kernel = SMAT_KERNEL_ROWWISE;
     }
+    // a plan made for a wide N, used with a narrow one: too few workgroups for the sweep kernel
+    if (kernel == SMAT_KERNEL_SWEEP && o.kernel == SMAT_KERNEL_AUTO && !sweep_fills_device(M / 16, N))
+        kernel = SMAT_KERNEL_ROWWISE;
     if (o.b_layout == SMAT_B_ROW_MAJOR && kernel != SMAT_KERNEL_COMPACT)
         return set_error(SMAT_ERR_UNSUPPORTED,
                          "row-major B (B[k*N+n]) is implemented for SMAT_KERNEL_COMPACT only; the other kernels "
@@ -238,12 +249,13 @@ extern "C" int smat_plan_create(smat_plan **out, const int32_t *row_ptr_host,
     }
     // The sweep kernel pays one pass over the B panel per group of 32 block rows,
     // whatever the sparsity, and shares each staged slab between the blocks of the group
-    // that sit in that block column.  At 10% of the blocks present (8192 x 8192, N = 4096) it
-    // takes 160 us against 173 us for the row-wise kernel on repacked B; its share of reused
-    // slabs grows with the density, the row-wise kernel's work does not shrink: taken from 9.5%.
+    // that sit in that block column.  Measured against the row-wise kernel on repacked B for
+    // M = K in {4096, 8192, 16384}, N in {512 .. 4096} and 5% .. 25% of the blocks present: it
+    // wins (by 1.02x at 5% up to 1.6x at 25%) whenever its workgroups (groups of 32 block
+    // rows x panels of 128 columns) fill the 256 CUs, and loses (0.3x .. 0.9x) when they do not.
     bool sweep = want == SMAT_KERNEL_SWEEP;
-    if (want == SMAT_KERNEL_AUTO && col_idx_host && n_hint >= 512 && mb >= 2 * (size_t)SWEEP_G &&
-        (double)nnzb >= 0.095 * (double)mb * (double)kb)
+    if (want == SMAT_KERNEL_AUTO && col_idx_host && sweep_fills_device(mb, n_hint) &&
+        (double)nnzb >= 0.05 * (double)mb * (double)kb)
         sweep = true;
     if (sweep && nnzb >= (size_t)1 << 23) { // the sweep kernel addresses blocks with 32-bit byte offsets
         if (want == SMAT_KERNEL_SWEEP) {
