@@ -268,6 +268,35 @@ def test_config5_stencil_reduced_and_reordered(smat, cuda, oracle):
     assert oracle.compare(C2, ref[pr])[0] <= TOL_F16
 
 
+def test_plan_takes_the_sweep_kernel_only_when_it_fills_the_device(smat, cuda, oracle):
+    import torch
+    # 64 groups of 32 block rows, 10 % of the blocks: 4 panels of 128 columns make 256 workgroups
+    A = gen.random_bcsr(2048, 32, 0.10, seed=77)
+    M, K, nnzb = A["M"], A["K"], A["nnzb"]
+    wide = smat.Plan(A["b_row_ptr"], M, K, nnzb, 512, col_idx_host=A["b_col_idx"])
+    narrow = smat.Plan(A["b_row_ptr"], M, K, nnzb, 384, col_idx_host=A["b_col_idx"])
+    assert wide.info()["kernel"] == SWEEP and narrow.info()["kernel"] == 1
+    narrow.close()
+    # too sparse (2 % of the blocks): row-wise whatever the width
+    S = gen.random_bcsr(2048, 32, 0.02, seed=78)
+    sparse = smat.Plan(S["b_row_ptr"], S["M"], S["K"], S["nnzb"], 512, col_idx_host=S["b_col_idx"])
+    assert sparse.info()["kernel"] == 1
+    sparse.close()
+    # the plan made for N = 512, used with N = 512 (sweep) and with N = 128 (falls back to row-wise)
+    vals, rp, ci = (to_dev(torch, A[k], cuda) for k in ("b_val", "b_row_ptr", "b_col_idx"))
+    for N in (512, 128):
+        B = gen.dense_b(K, N, seed=5 + N)
+        C = torch.full((M, N), 0x7E00, dtype=torch.int16, device=cuda)
+        smat.spmm(vals, rp, ci, to_dev(torch, B, cuda), C, M, N, K, nnzb, plan=wide)
+        torch.cuda.synchronize()
+        rows = slice(0, 16 * 40)
+        sub = {"M": 16 * 40, "K": K, "b_row_ptr": A["b_row_ptr"][:41], "b_col_idx": A["b_col_idx"][:A["b_row_ptr"][40]],
+               "b_val": A["b_val"][:A["b_row_ptr"][40] * 256]}
+        ref = oracle_ref(oracle, sub, B, N)
+        assert oracle.compare(C.cpu().numpy().view(np.uint16)[rows], ref)[0] <= TOL_F16
+    wide.close()
+
+
 def test_config4_block_pruned_full_size_sampled_rows(smat, cuda, oracle):
     A = gen.block_pruned(8192, 0.10, 0.02)
     assert A["nnzb"] == 26214
