@@ -68,7 +68,10 @@ int smat_spmm_bcsr_f16(const uint16_t *vals, const int32_t *row_ptr, const int32
 #define SMAT_KERNEL_AUTO 0
 #define SMAT_KERNEL_ROWWISE 1 /* one wavefront per (block-row chunk, N panel), operands straight from L2;
                                * the plan decides whether B is first repacked slab-major into scratch   */
-#define SMAT_KERNEL_SWEEP 2   /* workgroup sweeps K for a group of block rows, B panel staged in LDS      */
+#define SMAT_KERNEL_SWEEP 2   /* workgroup sweeps K for a group of 32 block rows x 128 columns, B panel staged
+                               * in LDS; needs a plan made with col_idx_host, fewer than 2^23 blocks and a B
+                               * smaller than 4 GiB.  SMAT_KERNEL_AUTO takes it when at least 5% of the blocks
+                               * exist and (M/512) x (N/128) workgroups fill the 256 CUs                     */
 #define SMAT_KERNEL_ROWWISE_DIRECT 3 /* row-wise, B always read in place (plan or launch option)          */
 #define SMAT_KERNEL_COMPACT 5  /* only the nonzero columns of the blocks are multiplied (needs
                                * smat_plan_attach_values); for blocks with few nonzero columns */
@@ -90,7 +93,8 @@ typedef struct smat_plan smat_plan;
 
 /* row_ptr_host: the HOST copy of the BCSR row pointer (M/16+1 entries).
  * col_idx_host: HOST copy of the BCSR column index (may be NULL unless
- *               opts->kernel requests SMAT_KERNEL_SWEEP).
+ *               opts->kernel requests SMAT_KERNEL_SWEEP; without it SMAT_KERNEL_AUTO
+ *               never chooses that kernel).
  * n_hint: the N the plan will mostly be used with (panel width choice). */
 int smat_plan_create(smat_plan **plan, const int32_t *row_ptr_host, const int32_t *col_idx_host,
                      size_t M, size_t K, size_t nnzb, size_t n_hint, const smat_spmm_opts *opts);
