@@ -30,7 +30,7 @@ PEAK_HBM_GBS = 8000.0      # MI355X HBM3E
 # HBM bytes per launch measured with rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE and scaled by a plain
 # device copy of known size (summaries under profiles/): (workload, kernel id) -> bytes
 MEASURED_TRAFFIC = {
-    ("block_pruned_8192_10pct_N4096", 2): 143442 * 1024 * 2.0 + 65824 * 1024 * 1.0,
+    ("block_pruned_8192_10pct_N4096", 2): 143436 * 1024 * 2.0 + 65972 * 1024 * 1.0,
     # row-wise kernel + repack kernel
     ("block_pruned_8192_10pct_N4096", 1): (247966 + 32783) * 1024 * 2.0 + (65538 + 65536) * 1024 * 1.0,
     # compact kernel + transpose kernel (+ reduce kernel for the split rows of R-MAT)
@@ -39,6 +39,13 @@ MEASURED_TRAFFIC = {
     ("stencil27_64_N64", 5): (70391 + 16399) * 1024 * 2.0 + (32768 + 32768) * 1024 * 1.0,
 }
 
+
+# Share of SIMD cycles with the MFMA pipe busy, rocprofv3 --pmc SQ_VALU_MFMA_BUSY_CYCLES / SQ_BUSY_CYCLES
+# (same summaries): informational, next to the roofline fraction
+MEASURED_MFMA_BUSY = {
+    ("block_pruned_8192_10pct_N4096", 2): 0.206,
+    ("block_pruned_8192_10pct_N4096", 1): 0.168,
+}
 
 INFO = {}  # facts about the generated workload that go into the config of the result line
 PERM_FILE = None
@@ -274,6 +281,8 @@ def main():
     if kernel_id == 1 and (plan is None or not plan.info()["b_pack_bytes"]):
         kernel_id = 3
     roof["traffic"] = MEASURED_TRAFFIC.get((args.workload, kernel_id))
+    if (args.workload, kernel_id) in MEASURED_MFMA_BUSY:
+        roof["mfma_busy_rocprof"] = MEASURED_MFMA_BUSY[(args.workload, kernel_id)]
     roof["kernel_ms"] = round(kernel_ms, 5)
     roof["algorithmic_flops"] = flops
     roof["algorithmic_bytes"] = qbytes
