@@ -193,6 +193,8 @@ SWEEP = 2
     (64, 33, 0.10, 256),    # K = 528: last chunk is 1 slab wide
     (33, 70, 0.05, 520),    # sparse enough that some (row group, chunk) records are empty
     (32, 16, 1.00, 128),    # fully dense: every op is a pair
+    (35, 3, 0.60, 8),       # narrowest N, K = 48: one partial chunk, most of the panel unused
+    (70, 20, 0.30, 72),     # N below one panel
 ])
 def test_sweep_kernel_matches_oracle(smat, cuda, oracle, mb, kb, density, N):
     A = gen.random_bcsr(mb, kb, density, seed=1000 + mb + kb)
