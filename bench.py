@@ -30,7 +30,7 @@ PEAK_HBM_GBS = 8000.0      # MI355X HBM3E
 # HBM bytes per launch measured with rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE and scaled by a plain
 # device copy of known size (summaries under profiles/): (workload, kernel id) -> bytes
 MEASURED_TRAFFIC = {
-    ("block_pruned_8192_10pct_N4096", 2): 143436 * 1024 * 2.0 + 65972 * 1024 * 1.0,
+    ("block_pruned_8192_10pct_N4096", 2): 143469 * 1024 * 2.0 + 66082 * 1024 * 1.0,
     # row-wise kernel + repack kernel
     ("block_pruned_8192_10pct_N4096", 1): (247966 + 32783) * 1024 * 2.0 + (65538 + 65536) * 1024 * 1.0,
     # compact kernel + transpose kernel (+ reduce kernel for the split rows of R-MAT)
@@ -43,7 +43,7 @@ MEASURED_TRAFFIC = {
 # Share of SIMD cycles with the MFMA pipe busy, rocprofv3 --pmc SQ_VALU_MFMA_BUSY_CYCLES / SQ_BUSY_CYCLES
 # (same summaries): informational, next to the roofline fraction
 MEASURED_MFMA_BUSY = {
-    ("block_pruned_8192_10pct_N4096", 2): 0.206,
+    ("block_pruned_8192_10pct_N4096", 2): 0.217,
     ("block_pruned_8192_10pct_N4096", 1): 0.168,
 }
 

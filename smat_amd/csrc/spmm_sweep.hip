@@ -20,11 +20,13 @@
 //    the table continues in a following record that reuses the resident B stage.
 //    A operands are 512-byte coalesced global reads straight into MFMA layout.
 //  * Software pipeline over chunks, everything for chunk c+1 is issued before the
-//    MFMA work of chunk c starts and is only waited for after it: the op table of
-//    chunk c+2, the A operands of chunk c+1 (into a second set of registers) and
-//    the B panel of chunk c+1 (global -> LDS asynchronously with
-//    global_load_lds_dwordx4, no staging registers, into the other LDS stage).
-//    The MFMA loop itself touches only registers and LDS.  One barrier per chunk.
+//    MFMA work of chunk c starts and is only waited for after it: the A operands of
+//    chunk c+1 (into a second set of registers) and the B panel of chunk c+1 (global
+//    -> LDS asynchronously with global_load_lds_dwordx4, no staging registers, into
+//    the other LDS stage).  The op table of chunk c+2 is requested right after the
+//    MFMA work of chunk c, into the registers of the table just used.  The loop is
+//    unrolled by two so that the two register sets swap roles without copies.  The
+//    MFMA loop itself touches only registers and LDS.  One barrier per chunk.
 //  * Vector memory instructions are the scarce resource of the load phase: the load
 //    path of a CU takes about one 64-lane instruction (up to 1 KiB) per 16 clocks and
 //    the issuing wavefront stalls meanwhile.  So the op tables are read with scalar
@@ -162,10 +164,14 @@ __global__ __launch_bounds__(THREADS) void spmm_sweep_kernel(
     // load path of the CU 16 clocks whatever it fetches.  The missing second block of a
     // single re-reads the first (zeroed at use).
     auto load_a = [&](f16x8 (&dst)[CAP], const u32x16 &tab) {
+        constexpr int CAPR = CAP / RW;
 #pragma unroll
-        for (int k = 0; k < CAP; k++) {
-            const uint32_t w0 = tab[2 * k], w1 = tab[2 * k + 1];
-            if (w0 != SWEEP_EMPTY_SLOT) {
+        for (int r = 0; r < RW; r++) {
+#pragma unroll
+            for (int j = 0; j < CAPR; j++) {
+                const int k = r * CAPR + j;
+                const uint32_t w0 = tab[2 * k], w1 = tab[2 * k + 1];
+                if (w0 == SWEEP_EMPTY_SLOT) break; // the slots of a block row fill up in order
                 const uint32_t b1 = (w0 & 0xFFFFFFu) * 512u; // nnzb < 2^23 is checked by the plan
                 const uint32_t p2 = w1 & 0xFFFFFFu;
                 const uint32_t b2 = p2 == SWEEP_NO_BLOCK ? b1 : p2 * 512u;
@@ -175,89 +181,89 @@ __global__ __launch_bounds__(THREADS) void spmm_sweep_kernel(
         }
     };
 
-    u32x16 tab_cur, tab_nxt, tab_nx2;
+    // Two sets of op-table registers and of A operand registers; consecutive records use
+    // them in swapped roles (the loop below is unrolled by two), so nothing is copied.
+    u32x16 tab0, tab1;
 #pragma unroll
-    for (int k = 0; k < 16; k++) { tab_cur[k] = SWEEP_EMPTY_SLOT; tab_nxt[k] = SWEEP_EMPTY_SLOT; tab_nx2[k] = SWEEP_EMPTY_SLOT; }
-
-    f16x8 a_cur[CAP], a_nxt[CAP];
+    for (int k = 0; k < 16; k++) { tab0[k] = SWEEP_EMPTY_SLOT; tab1[k] = SWEEP_EMPTY_SLOT; }
+    f16x8 a0[CAP], a1[CAP];
 #pragma unroll
-    for (int k = 0; k < CAP; k++) { a_cur[k] = zero8; a_nxt[k] = zero8; }
+    for (int k = 0; k < CAP; k++) { a0[k] = zero8; a1[k] = zero8; }
 
     int stage = 0;
+    const int last = c_end - 1;
     if (c_begin < c_end) {
-        const int last = c_end - 1;
-        tab_cur = load_op_table(ops, c_begin, wave);
-        tab_nxt = load_op_table(ops, c_begin + 1 < last ? c_begin + 1 : last, wave);
+        tab0 = load_op_table(ops, c_begin, wave);
+        tab1 = load_op_table(ops, c_begin + 1 < last ? c_begin + 1 : last, wave);
         fill_issue(lds, B, chunk_ids[c_begin] & ~SWEEP_CONT_FLAG, n0, N, K, wave, lane);
-        load_a(a_cur, tab_cur);
+        load_a(a0, tab0);
     }
     __builtin_amdgcn_s_waitcnt(0x0f70); // vmcnt(0): the copies of this wavefront have landed
     __syncthreads();
 
-    for (int ci = c_begin; ci < c_end; ci++) {
-        const int last = c_end - 1;
+    // One record: tab_c / a_c hold the op table and A operands of record ci, tab_n the table of
+    // record ci + 1, whose A operands go to a_n.
+    auto record = [&](int ci, u32x16 &tab_c, const u32x16 &tab_n, f16x8 (&a_c)[CAP], f16x8 (&a_n)[CAP]) {
+        // ---- everything record ci+1 needs ----
         bool next_is_new = false;
-        // ---- everything chunk ci+1 (and the table of ci+2) needs ----
-        // Past the end the last record's table is simply loaded again.
-        auto do_loads = [&]() {
-            tab_nx2 = load_op_table(ops, ci + 2 < last ? ci + 2 : last, wave);
-            if (ci + 1 < c_end) {
-                load_a(a_nxt, tab_nxt);
-                // A record that continues the chunk of the previous record (its ops did not
-                // fit one table) has bit 30 set: no B copy, the LDS stage stays.
-                const int next_chunk = chunk_ids[ci + 1];
-                next_is_new = !(next_chunk & SWEEP_CONT_FLAG);
-                if (next_is_new)
-                    fill_issue(lds + (stage ^ 1) * STAGE_BYTES, B, next_chunk, n0, N, K, wave, lane);
-            }
-        };
-        // ---- MFMA work of chunk ci: registers and LDS only ----
-        auto do_compute = [&]() {
-            const unsigned char *cur = lds + stage * STAGE_BYTES + rd_base;
+        if (ci + 1 < c_end) {
+            load_a(a_n, tab_n);
+            // A record that continues the chunk of the previous record (its ops did not
+            // fit one table) has bit 30 set: no B copy, the LDS stage stays.
+            const int next_chunk = chunk_ids[ci + 1];
+            next_is_new = !(next_chunk & SWEEP_CONT_FLAG);
+            if (next_is_new)
+                fill_issue(lds + (stage ^ 1) * STAGE_BYTES, B, next_chunk, n0, N, K, wave, lane);
+        }
+        // ---- MFMA work of record ci: registers and LDS only ----
+        const unsigned char *cur = lds + stage * STAGE_BYTES + rd_base;
 #pragma unroll
-            for (int k = 0; k < CAP; k++) {
-                // slot k belongs to block row k / CAPR of this wavefront: the accumulator
-                // registers of every slot are fixed at compile time
-                constexpr int CAPR = CAP / RW;
-                const uint32_t w0 = tab_cur[2 * k], w1 = tab_cur[2 * k + 1];
-                if (w0 != SWEEP_EMPTY_SLOT) {
-                    const uint32_t soff = sel ? slab_offset(w1 >> 24) : slab_offset(w0 >> 24);
-                    const unsigned char *bp = cur + (soff ^ lane_xor);
-                    f16x8 av = a_cur[k];
-                    if ((w1 & 0xFFFFFFu) == SWEEP_NO_BLOCK) // single: no second block
-                        av = sel ? zero8 : av;
+        for (int r = 0; r < RW; r++) {
+            // table slot k belongs to block row k / CAPR of this wavefront: the accumulator
+            // registers of every slot are fixed at compile time
+            constexpr int CAPR = CAP / RW;
 #pragma unroll
-                    for (int u = 0; u < TN / 4; u++) {
-                        f16x8 b[4];
+            for (int j = 0; j < CAPR; j++) {
+                const int k = r * CAPR + j;
+                const uint32_t w0 = tab_c[2 * k], w1 = tab_c[2 * k + 1];
+                if (w0 == SWEEP_EMPTY_SLOT) break; // the slots of a block row fill up in order
+                const uint32_t soff = sel ? slab_offset(w1 >> 24) : slab_offset(w0 >> 24);
+                const unsigned char *bp = cur + (soff ^ lane_xor);
+                f16x8 av = a_c[k];
+                if ((w1 & 0xFFFFFFu) == SWEEP_NO_BLOCK) // single: no second block
+                    av = sel ? zero8 : av;
 #pragma unroll
-                        for (int tt = 0; tt < 4; tt++)
-                            b[tt] = *reinterpret_cast<const f16x8 *>(bp + (64 * u + 4 * tt) * ROW_BYTES);
+                for (int u = 0; u < TN / 4; u++) {
+                    f16x8 b[4];
 #pragma unroll
-                        for (int tt = 0; tt < 4; tt++)
-                            acc[k / CAPR][u * 4 + tt] = __builtin_amdgcn_mfma_f32_16x16x32_f16(
-                                b[tt], av, acc[k / CAPR][u * 4 + tt], 0, 0, 0);
-                    }
-                    // order of the 8 LDS reads and 8 MFMAs of this op: four reads ahead, then one
-                    // MFMA per further read, so an MFMA never waits on the read issued just before it
-                    __builtin_amdgcn_sched_group_barrier(0x100, 4, 0);
+                    for (int tt = 0; tt < 4; tt++)
+                        b[tt] = *reinterpret_cast<const f16x8 *>(bp + (64 * u + 4 * tt) * ROW_BYTES);
 #pragma unroll
-                    for (int q = 0; q < 4; q++) {
-                        __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
-                        __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);
-                    }
-                    __builtin_amdgcn_sched_group_barrier(0x008, 4, 0);
+                    for (int tt = 0; tt < 4; tt++)
+                        acc[r][u * 4 + tt] = __builtin_amdgcn_mfma_f32_16x16x32_f16(
+                            b[tt], av, acc[r][u * 4 + tt], 0, 0, 0);
                 }
+                // order of the 8 LDS reads and 8 MFMAs of this op: four reads ahead, then one
+                // MFMA per further read, so an MFMA never waits on the read issued just before it
+                __builtin_amdgcn_sched_group_barrier(0x100, 4, 0);
+#pragma unroll
+                for (int q = 0; q < 4; q++) {
+                    __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
+                    __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);
+                }
+                __builtin_amdgcn_sched_group_barrier(0x008, 4, 0);
             }
-        };
-        do_loads();
-        do_compute();
-        __builtin_amdgcn_s_waitcnt(0x0f70); // vmcnt(0): next chunk's B, A and table have landed
+        }
+        // the table of record ci+2 replaces the one just used (a scalar load: it returns
+        // while this wavefront waits for the copies and at the barrier)
+        if (ci + 2 <= last) tab_c = load_op_table(ops, ci + 2, wave);
+        __builtin_amdgcn_s_waitcnt(0x0f70); // vmcnt(0): next record's B and A have landed
         __syncthreads();
         if (next_is_new) stage ^= 1;
-        tab_cur = tab_nxt;
-        tab_nxt = tab_nx2;
-#pragma unroll
-        for (int k = 0; k < CAP; k++) a_cur[k] = a_nxt[k];
+    };
+    for (int ci = c_begin; ci < c_end; ci += 2) {
+        record(ci, tab0, tab1, a0, a1);
+        if (ci + 1 < c_end) record(ci + 1, tab1, tab0, a1, a0);
     }
     // Epilogue: acc[r][t][e] = C[(rg*G + wave*RW + r)*16 + i16][n0 + 64*(t/4) + 16*g + 4*(t%4) + e]
 #pragma unroll
