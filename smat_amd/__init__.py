@@ -7,6 +7,12 @@ missing, loading raises.
 """
 from ._lib import lib, SmatError, library_path  # noqa: F401
 from .host import (  # noqa: F401
+    KERNEL_AUTO,
+    KERNEL_ROWWISE,
+    KERNEL_SWEEP,
+    KERNEL_ROWWISE_DIRECT,
+    KERNEL_ROWWISE_PACKED,
+    KERNEL_COMPACT,
     Bcsr,
     Plan,
     csr_to_bcsr,
@@ -26,4 +32,5 @@ from .host import (  # noqa: F401
 __all__ = [
     "lib", "SmatError", "library_path", "Bcsr", "Plan", "csr_to_bcsr", "bin_write_csr", "bin_write_bcsr", "bin_read", "mtx_write", "csr_to_bcsr_device", "DeviceBcsr", "mtx_read",
     "permute_csr", "reorder_csr", "reorder_rows", "spmm",
+    "KERNEL_AUTO", "KERNEL_ROWWISE", "KERNEL_SWEEP", "KERNEL_ROWWISE_DIRECT", "KERNEL_ROWWISE_PACKED", "KERNEL_COMPACT",
 ]
