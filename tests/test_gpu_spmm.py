@@ -224,6 +224,20 @@ def test_sweep_needs_a_plan_with_col_idx(smat, cuda):
         smat.Plan(A["b_row_ptr"], A["M"], A["K"], A["nnzb"], 128, col_idx_host=None, kernel=SWEEP)
 
 
+def test_sweep_refuses_a_b_of_4_gib_or_more(smat, cuda):
+    """The sweep kernel addresses B with 32-bit byte offsets: an explicit request is refused before any
+    launch (the buffers here are dummies that are never touched)."""
+    import torch
+    M, K, N = 16, 65536, 32768  # K * N * 2 bytes = 4 GiB
+    rp = np.array([0, 1], np.int32)
+    ci = np.array([0], np.int32)
+    plan = smat.Plan(rp, M, K, 1, 128, col_idx_host=ci, kernel=SWEEP)
+    dummy = torch.zeros(4096, dtype=torch.int16, device=cuda)
+    with pytest.raises(smat.SmatError):
+        smat.spmm(dummy, to_dev(torch, rp, cuda), to_dev(torch, ci, cuda), dummy, dummy, M, N, K, 1, plan=plan, kernel=SWEEP)
+    plan.close()
+
+
 def test_b_ones_gives_row_sums(smat, cuda, oracle):
     # the reference fills B with 1.0 (common/matrix.h:38): every column of C is the row sum of A
     A = gen.random_bcsr(12, 12, 0.4, seed=77)
