@@ -117,7 +117,12 @@ int smat_plan_info(const smat_plan *plan, int64_t *info);
 
 /* Same operands as smat_spmm_bcsr_f16; C is uint16_t* or float* per opts->c_dtype.
  * opts == NULL means defaults; plan == NULL means no work list (whole block
- * rows, one wavefront each). */
+ * rows, one wavefront each).
+ * Non-finite inputs: an unpaired block is multiplied together with a block of zeros
+ * (one MFMA covers two blocks) and the compact kernel pads a block row with zero
+ * columns; 0 x Inf = NaN, so where B holds Inf or NaN a result element can come out
+ * NaN where a block-by-block product (mmaCBT.cu:44-66) gives Inf.  Finite inputs give
+ * the same sums up to the fp32 summation order. */
 int smat_spmm_bcsr_f16_ex(const uint16_t *vals, const int32_t *row_ptr, const int32_t *col_idx,
                           const uint16_t *B, void *C, size_t M, size_t N, size_t K, size_t nnzb,
                           const smat_spmm_opts *opts, const smat_plan *plan);
