@@ -13,6 +13,7 @@
 #include "../../include/smat.h"
 #include "errors.h"
 #include "spmm_kernels.h"
+#include "sweep_plan.h"
 
 using namespace smat;
 
@@ -38,7 +39,7 @@ struct smat_plan {
     uint16_t *d_bpack = nullptr; // slab-major copy of B, K * n_cap halves (row-wise kernel, when it pays)
     // sweep kernel work list (present when kernel == SMAT_KERNEL_SWEEP)
     int n_rg = 0, n_records = 0, n_ops = 0;
-    int32_t *d_rg_chunk_ptr = nullptr, *d_chunk_ids = nullptr;
+    int32_t *d_rg_chunk_ptr = nullptr, *d_chunk_ids = nullptr, *d_op_ptr = nullptr;
     SweepOp *d_ops = nullptr;
     // compacted-column kernel (present after smat_plan_attach_values)
     CompactPlan *compact = nullptr;
@@ -65,7 +66,7 @@ static int check_shapes(const void *vals, const void *row_ptr, const void *col_i
     return SMAT_OK;
 }
 
-// The sweep kernel runs one workgroup per (group of SWEEP_G block rows, panel of 128 columns),
+// The sweep kernel runs one workgroup per (group of SWEEP_G block rows, panel of 64 columns),
 // one workgroup per CU at a time.
 static bool sweep_fills_device(size_t mb, size_t n)
 {
@@ -115,9 +116,9 @@ extern "C" int smat_spmm_bcsr_f16_ex(const uint16_t *vals, const int32_t *row_pt
     if (kernel != SMAT_KERNEL_ROWWISE && kernel != SMAT_KERNEL_SWEEP && kernel != SMAT_KERNEL_COMPACT)
         return set_error(SMAT_ERR_INVALID, "unknown kernel id %d", kernel);
     hipError_t e;
-    if (kernel == SMAT_KERNEL_SWEEP && K * N >= ((size_t)1 << 31)) { // its B copies use 32-bit byte offsets
+    if (kernel == SMAT_KERNEL_SWEEP && K >= ((size_t)1 << 28)) { // its B copies use 32-bit offsets inside four columns
         if (o.kernel == SMAT_KERNEL_SWEEP)
-            return set_error(SMAT_ERR_UNSUPPORTED, "SMAT_KERNEL_SWEEP takes a B smaller than 4 GiB");
+            return set_error(SMAT_ERR_UNSUPPORTED, "SMAT_KERNEL_SWEEP takes K below 2^28");
         kernel = SMAT_KERNEL_ROWWISE;
     }
     // a plan made for a wide N, used with a narrow one: too few workgroups for the sweep kernel
@@ -139,9 +140,9 @@ extern "C" int smat_spmm_bcsr_f16_ex(const uint16_t *vals, const int32_t *row_pt
         if (!plan || !plan->d_ops)
             return set_error(SMAT_ERR_INVALID, "SMAT_KERNEL_SWEEP needs a plan built for it (with col_idx_host)");
         SweepArgs w{};
-        w.vals = vals; w.B = B; w.C = C; w.M = M; w.N = N; w.K = K; w.c_f32 = a.c_f32;
+        w.vals = vals; w.B = B; w.C = C; w.M = M; w.N = N; w.K = K; w.nnzb = nnzb; w.c_f32 = a.c_f32;
         w.rg_chunk_ptr = plan->d_rg_chunk_ptr; w.chunk_ids = plan->d_chunk_ids;
-        w.ops = plan->d_ops; w.n_rg = plan->n_rg;
+        w.op_ptr = plan->d_op_ptr; w.ops = plan->d_ops; w.n_rg = plan->n_rg;
         e = launch_sweep(w, static_cast<hipStream_t>(o.stream));
     } else {
         e = launch_rowwise(a, static_cast<hipStream_t>(o.stream));
@@ -257,89 +258,31 @@ extern "C" int smat_plan_create(smat_plan **out, const int32_t *row_ptr_host,
     if (want == SMAT_KERNEL_AUTO && col_idx_host && sweep_fills_device(mb, n_hint) &&
         (double)nnzb >= 0.05 * (double)mb * (double)kb)
         sweep = true;
-    if (sweep && nnzb >= (size_t)1 << 23) { // the sweep kernel addresses blocks with 32-bit byte offsets
+    if (sweep && (nnzb >= (size_t)1 << 23 || nnzb < 2)) { // blocks are addressed in pairs, with 32-bit byte offsets
         if (want == SMAT_KERNEL_SWEEP) {
             smat_plan_destroy(p);
-            return set_error(SMAT_ERR_UNSUPPORTED, "SMAT_KERNEL_SWEEP supports fewer than 2^23 nonzero blocks");
+            return set_error(SMAT_ERR_UNSUPPORTED, "SMAT_KERNEL_SWEEP takes between 2 and 2^23 - 1 nonzero blocks");
         }
         sweep = false;
     }
     if (e == hipSuccess && sweep) {
-        const size_t n_rg = (mb + SWEEP_G - 1) / SWEEP_G;
-        std::vector<int32_t> rg_ptr(n_rg + 1, 0), chunk_ids;
-        std::vector<SweepOp> ops; // records * SWEEP_WAVES * SWEEP_CAP table slots
-        const SweepOp empty_slot = {SWEEP_EMPTY_SLOT, SWEEP_EMPTY_SLOT};
-        struct Ent { int32_t chunk, wave, r, slab, p; };
-        std::vector<Ent> ents;
-        constexpr int CAPR = SWEEP_CAP / SWEEP_RW; // table slots per block row
-        std::vector<SweepOp> per_row[SWEEP_WAVES][SWEEP_RW];
-        size_t n_ops = 0;
-        for (size_t rg = 0; rg < n_rg; rg++) {
-            ents.clear();
-            const size_t r_end = std::min(mb, (rg + 1) * SWEEP_G);
-            for (size_t br = rg * SWEEP_G; br < r_end; br++) {
-                const int local = (int)(br - rg * SWEEP_G);
-                for (int32_t q = row_ptr_host[br]; q < row_ptr_host[br + 1]; q++) {
-                    const int32_t bc = col_idx_host[q] / 16;
-                    ents.push_back(Ent{bc / SWEEP_S, local / SWEEP_RW, local % SWEEP_RW, bc % SWEEP_S, q});
-                }
-            }
-            std::sort(ents.begin(), ents.end(), [](const Ent &x, const Ent &y) {
-                if (x.chunk != y.chunk) return x.chunk < y.chunk;
-                if (x.wave != y.wave) return x.wave < y.wave;
-                if (x.r != y.r) return x.r < y.r;
-                return x.slab < y.slab;
-            });
-            size_t i = 0;
-            while (i < ents.size()) {
-                const int32_t chunk = ents[i].chunk;
-                size_t most = 0;
-                for (int w = 0; w < SWEEP_WAVES; w++)
-                    for (int r = 0; r < SWEEP_RW; r++) {
-                        std::vector<SweepOp> &list = per_row[w][r];
-                        list.clear();
-                        while (i < ents.size() && ents[i].chunk == chunk && ents[i].wave == w && ents[i].r == r) {
-                            const bool pair = i + 1 < ents.size() && ents[i + 1].chunk == chunk &&
-                                              ents[i + 1].wave == w && ents[i + 1].r == r;
-                            SweepOp op;
-                            op.w0 = (uint32_t)ents[i].p | ((uint32_t)ents[i].slab << 24);
-                            // a single block: the upper MFMA half gets zeros of A and reads the same slab
-                            op.w1 = pair ? ((uint32_t)ents[i + 1].p | ((uint32_t)ents[i + 1].slab << 24))
-                                         : (SWEEP_NO_BLOCK | ((uint32_t)ents[i].slab << 24));
-                            list.push_back(op);
-                            i += pair ? 2 : 1;
-                        }
-                        most = std::max(most, list.size());
-                        n_ops += list.size();
-                    }
-                // one record per CAPR ops of the busiest block row; records after the first
-                // reuse the B stage that is already resident
-                const size_t n_rec = (most + CAPR - 1) / CAPR;
-                for (size_t rec = 0; rec < n_rec; rec++) {
-                    chunk_ids.push_back(rec == 0 ? chunk : (chunk | SWEEP_CONT_FLAG));
-                    for (int w = 0; w < SWEEP_WAVES; w++)
-                        for (int r = 0; r < SWEEP_RW; r++)
-                            for (int j = 0; j < CAPR; j++) {
-                                const size_t idx = rec * CAPR + j;
-                                ops.push_back(idx < per_row[w][r].size() ? per_row[w][r][idx] : empty_slot);
-                            }
-                }
-            }
-            rg_ptr[rg + 1] = (int32_t)chunk_ids.size();
-        }
+        SweepPlanHost h;
+        build_sweep_plan(row_ptr_host, col_idx_host, mb, kb, h);
         p->kernel = SMAT_KERNEL_SWEEP;
-        p->n_rg = (int)n_rg;
-        p->n_records = (int)chunk_ids.size();
-        p->n_ops = (int)n_ops;
+        p->n_rg = (int)h.rg_chunk_ptr.size() - 1;
+        p->n_records = (int)h.chunk_ids.size();
+        p->n_ops = (int)(h.ops.size() - SWEEP_OP_PAD);
         auto upload = [&](void **dst, const void *src, size_t bytes) {
             if (e != hipSuccess) return;
             e = hipMalloc(dst, std::max<size_t>(bytes, 16));
             if (e == hipSuccess && bytes) e = hipMemcpy(*dst, src, bytes, hipMemcpyHostToDevice);
         };
-        upload((void **)&p->d_rg_chunk_ptr, rg_ptr.data(), rg_ptr.size() * sizeof(int32_t));
-        upload((void **)&p->d_chunk_ids, chunk_ids.data(), chunk_ids.size() * sizeof(int32_t));
-        upload((void **)&p->d_ops, ops.data(), ops.size() * sizeof(SweepOp));
-        if (p->d_bpack && want == SMAT_KERNEL_AUTO) { // the sweep kernel reads B in place
+        upload((void **)&p->d_rg_chunk_ptr, h.rg_chunk_ptr.data(), h.rg_chunk_ptr.size() * sizeof(int32_t));
+        upload((void **)&p->d_chunk_ids, h.chunk_ids.data(), h.chunk_ids.size() * sizeof(int32_t));
+        upload((void **)&p->d_op_ptr, h.op_ptr.data(), h.op_ptr.size() * sizeof(int32_t));
+        static_assert(sizeof(SweepOpHost) == sizeof(SweepOp), "host and device op layouts");
+        upload((void **)&p->d_ops, h.ops.data(), h.ops.size() * sizeof(SweepOp));
+        if (p->d_bpack && want != SMAT_KERNEL_ROWWISE_PACKED) { // the sweep kernel reads B in place
             (void)hipFree(p->d_bpack);
             p->d_bpack = nullptr;
         }
@@ -397,6 +340,7 @@ extern "C" int smat_plan_destroy(smat_plan *p)
     if (p->d_bpack) (void)hipFree(p->d_bpack);
     if (p->d_rg_chunk_ptr) (void)hipFree(p->d_rg_chunk_ptr);
     if (p->d_chunk_ids) (void)hipFree(p->d_chunk_ids);
+    if (p->d_op_ptr) (void)hipFree(p->d_op_ptr);
     if (p->d_ops) (void)hipFree(p->d_ops);
     delete p;
     return SMAT_OK;

@@ -1,42 +1,42 @@
-// "Sweep" SpMM kernel for block matrices that are dense enough (a few percent of
-// the 16x16 blocks present) and wide N: one workgroup owns a group of 32 block
-// rows x 128 columns of C and sweeps over K in chunks of 16 block columns.
+// "Sweep" SpMM kernel for block matrices that are dense enough (a few percent of the 16x16 blocks
+// present) and wide N.  One workgroup (8 wavefronts) owns 64 block rows x 64 columns of C and sweeps
+// over K in chunks of 16 block columns.
 //
-//  * The B panel of a chunk (256 k x 128 n, 64 KiB) is staged once per workgroup
-//    in LDS and shared by all block rows of the group; global reads of it are
-//    256-byte contiguous runs of the column-major B (B[n*K + k]), i.e. fully
-//    used cache lines, instead of the 32-byte gathers a per-block read costs.
-//  * LDS holds a chunk as [8-slab group][n][16 slots of 16 B]; a slot is 8
-//    consecutive k of one n.  The slot index is XOR-ed with a 4-bit function of
-//    n chosen so that the 16 lanes of one ds_read_b128 phase (which read 16
-//    different n, same logical slot) hit 16 different 16-byte bank groups, and
-//    the 16 lanes that fill one n write 256 contiguous bytes: no bank conflicts
-//    on either side.
-//  * Each wavefront owns 4 block rows (128 fp32 accumulator registers) and runs
-//    a host-built table of MFMA ops with a fixed number of slots per block row
-//    (so the accumulator registers of every slot are known at compile time):
-//    pairs of blocks of one block row inside the chunk feed one
-//    v_mfma_f32_16x16x32_f16 (K = 32 = 2 blocks).  A chunk whose ops do not fit
-//    the table continues in a following record that reuses the resident B stage.
-//    A operands are 512-byte coalesced global reads straight into MFMA layout.
-//  * Software pipeline over chunks, everything for chunk c+1 is issued before the
-//    MFMA work of chunk c starts and is only waited for after it: the A operands of
-//    chunk c+1 (into a second set of registers) and the B panel of chunk c+1 (global
-//    -> LDS asynchronously with global_load_lds_dwordx4, no staging registers, into
-//    the other LDS stage).  The op table of chunk c+2 is requested right after the
-//    MFMA work of chunk c, into the registers of the table just used.  The loop is
-//    unrolled by two so that the two register sets swap roles without copies.  The
-//    MFMA loop itself touches only registers and LDS.  One barrier per chunk.
-//  * Vector memory instructions are the scarce resource of the load phase: the load
-//    path of a CU takes about one 64-lane instruction (up to 1 KiB) per 16 clocks and
-//    the issuing wavefront stalls meanwhile.  So the op tables are read with scalar
-//    loads (64 bytes per record and wavefront), empty table slots load no A, and the
-//    B copies move 16 bytes per lane from a scalar base plus a 32-bit lane offset.
+//  * B.  The panel of a chunk (256 k x 64 n, 32 KiB) is copied global -> LDS asynchronously
+//    (global_load_lds_dwordx4, no staging registers) into a ring of four stages and is shared by the
+//    64 block rows.  Global reads are 256-byte contiguous runs of the column-major B (B[n*K + k]).
+//    A stage is [8-slab group][n][16 slots of 16 B]; a slot is 8 consecutive k of one n.  The slot
+//    index is XOR-ed with a 4-bit function of n so that the 16 lanes of one ds_read_b128 phase
+//    (16 different n, same logical slot) hit 16 different 16-byte bank groups and the 16 lanes that
+//    fill one n write 256 contiguous bytes: no bank conflicts on either side.
+//  * Work.  A wavefront owns 8 block rows x 64 columns (128 fp32 accumulator registers) and runs a
+//    host-built stream of ops.  One op = two blocks of one block row = one K = 32 step of
+//    v_mfma_f32_16x16x32_f16 per 16 columns (4 MFMAs).  The two blocks may sit in the same chunk or
+//    in two consecutive chunks (the ring keeps the previous stage), so few blocks stay unpaired; an
+//    unpaired block multiplies zeros in the upper K half.
+//  * Pipeline.  The op stream of a wavefront is one flat loop over the whole K sweep, unrolled by
+//    six: the B operands of an op are read from LDS two ops ahead (three register sets), its A
+//    operand (two neighbouring 512-byte blocks, one load straight into MFMA layout) comes from global
+//    memory four ops ahead (ring of six), its descriptor (16 bytes, offsets ready to use) is read
+//    six ops ahead from a window of the op stream that is itself copied into LDS 64 ops at a time.
+//    LDS reads are ordinary loads (the compiler counts them); everything that goes through the
+//    vector memory path (A loads, copies) is issued from inline assembly with explicit s_waitcnt
+//    vmcnt, because only the kernel knows which copies an A load does not have to wait for: vector
+//    memory instructions complete in order, and the number of younger ones is known at every wait.
+//  * Accumulators live in a[0:127] and are touched by inline assembly only: the block row of an op
+//    is a run-time value, and the choice between register sets is a branch between MFMA groups.
+//  * Synchronisation.  One barrier per chunk.  Entering chunk c: the copies of chunk c+1 (issued one
+//    chunk earlier) have landed, barrier, then the copies of chunk c+2 are issued into the stage
+//    that held chunk c-2.  Reads may therefore run ahead into chunk c+1 across the barrier.  The
+//    plan gives every wavefront at least two ops per chunk (zero-valued filler ops where a
+//    wavefront has fewer), so an op two ahead is never further than the next chunk and every
+//    wavefront passes every barrier.
 //
-// Same operand semantics as the reference launcher
-// (src/cuda_hgemm/src/mma/mmaCBT.cu:83-88).
+// Same operand semantics as the reference launcher (src/cuda_hgemm/src/mma/mmaCBT.cu:83-88).
 #include <hip/hip_runtime.h>
 #include <stdint.h>
+
+#include <type_traits>
 
 #include "spmm_kernels.h"
 
@@ -44,270 +44,359 @@ namespace smat {
 
 typedef _Float16 f16x8 __attribute__((ext_vector_type(8)));
 typedef float f32x4 __attribute__((ext_vector_type(4)));
+typedef int i32x4 __attribute__((ext_vector_type(4)));
 
 namespace {
 
-constexpr int TN = SWEEP_TN, RW = SWEEP_RW, W = SWEEP_WAVES, S = SWEEP_S;
-constexpr int NT = 16 * TN;                 // 128 columns per panel
-constexpr int THREADS = 64 * W;             // 512
-constexpr int OCTS = S / 8;                 // 8-slab groups per chunk
-constexpr int ROW_BYTES = 256;              // 8 slabs x 16 k x 2 B per n
-constexpr int STAGE_BYTES = OCTS * NT * ROW_BYTES; // 65536
-constexpr int FILL_ITERS = STAGE_BYTES / 16 / THREADS; // 16-byte slots per thread per chunk: 8
+constexpr int TN = SWEEP_TN, RW = SWEEP_RW, W = SWEEP_WAVES, S = SWEEP_S, NS = SWEEP_STAGES;
+constexpr int NT = 16 * TN;                           // 64 columns per panel
+constexpr int THREADS = 64 * W;                       // 512
+constexpr int ROW_BYTES = 256;                        // 8 slabs x 16 k x 2 B per n
+constexpr int STAGE_BYTES = (S / 8) * NT * ROW_BYTES; // 32768
+constexpr int COPIES = STAGE_BYTES / 1024 / W;        // copy instructions per wavefront and chunk: 4
+constexpr int PB = 2;                                 // B operands are read PB ops ahead (PB + 1 register sets)
+constexpr int DA = 6;                                 // A operand ring (register sets)
+constexpr int AHEAD = 4;                              // A operands are loaded AHEAD ops ahead (< DA)
+constexpr int DQ = 6;                                 // op descriptors are read from LDS DQ ops ahead (ring of DQ scalar pairs)
+constexpr int UNROLL = 6;                             // multiple of PB + 1, DA and DQ
+constexpr int WIN_SLOTS = 3;                          // descriptor windows (64 ops, 1 KiB) resident per wavefront
+constexpr int WINDOW_BYTES = W * WIN_SLOTS * 1024;    // 24 KiB
+static_assert(TN == 4 && RW == 8 && W == 8 && S == 16 && NS == 4 && COPIES == 4, "geometry the code below assumes");
+static_assert(UNROLL % (PB + 1) == 0 && UNROLL % DA == 0 && UNROLL % DQ == 0 && AHEAD < DA && AHEAD < DQ && PB < DQ,
+              "register sets are addressed by the unroll position");
 
-// LDS slot swizzle: physical slot = logical slot ^ ((n & 3) | ((n >> 2) & 12)), n = column in the panel.
-
-// Issues the asynchronous global -> LDS copies of one chunk of the B panel into
-// `stage`.  One wave instruction moves 64 x 16 B = 1 KiB: four n-rows of 256 B.
-// LDS destination = wave-uniform base + lane * 16 (hardware addressing of
-// global_load_lds_dwordx4); the global source is per lane, so the XOR swizzle is
-// applied on the source side.  Columns beyond N are skipped (their LDS rows only
-// feed C columns that are never stored) and k is clamped into the matrix (slabs
-// past K are referenced by no op).
-__device__ __forceinline__ void fill_issue(unsigned char *stage, const uint16_t *__restrict__ B,
-                                           int chunk, int n0, int N, long K, int wave, int lane)
+__device__ __forceinline__ void zero_accumulators()
 {
-    // Instruction `it` of wavefront `wave` covers rows (it*W + wave)*4 .. +3 of the
-    // stage, i.e. slab group o = it/4 and n = (it%4)*32 + wave*4 + lane/16.
-    static_assert(W == 8 && NT == 128 && FILL_ITERS == 8, "fill mapping assumes 8 waves x 128 columns");
-    const int q = lane >> 4, ps = lane & 15;
-    // swizzle_of_n(n) = q | bit4(n) << 2 | bit5(n) << 3 with bit4(n) = wave/4, bit5(n) = it & 1
-    const int ls0 = ps ^ (q | (((wave >> 2) & 1) << 2));
-    // Source address = wave-uniform base (column block of the instruction) + 32-bit lane
-    // offset: the launcher checks that B is smaller than 4 GiB.
-    const uint32_t kmax = (uint32_t)K - 8u;
-    const uint32_t col_off = (uint32_t)(n0 + wave * 4 + q) * (uint32_t)K; // in elements
-    const uint32_t k0 = (uint32_t)chunk * (S * 16);
-#pragma unroll
-    for (int it = 0; it < FILL_ITERS; it++) {
-        const int nrow = n0 + (it & 3) * 32 + wave * 4; // first of 4 columns, wave-uniform
-        if (nrow >= N) continue;                          // N % 8 == 0: all four or none
-        const uint32_t ls = (uint32_t)(ls0 ^ ((it & 1) << 3));
-        uint32_t k = k0 + (it >> 2) * 128 + ls * 8;
-        k = k < kmax ? k : kmax; // slabs past K are never referenced; keep the read in bounds
-        const uint32_t voff = (col_off + k) * 2u;
-        const uint16_t *sbase = B + (long)((it & 3) * 32) * K;
-        // Issued from inline assembly on purpose: the compiler orders every later LDS
-        // read after a global->LDS copy it knows about (it cannot tell the two stages
-        // apart) and would wait for the copy before the MFMA work of the current
-        // chunk.  The copies are waited for explicitly (vmcnt(0)) before the barrier.
-        const uint32_t dst = (uint32_t)(uintptr_t)(__attribute__((address_space(3))) void *)(
-            stage + (size_t)(it * W + wave) * 1024);
-        asm volatile("s_mov_b32 m0, %2\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, %1"
-                     :
-                     : "v"(voff), "s"(sbase), "s"(dst)
-                     : "memory", "m0");
-    }
+#define Z4(b) "v_accvgpr_write_b32 a" #b ", 0\n\t"
+#define Z16(b0, b1, b2, b3, b4, b5, b6, b7, b8, b9, b10, b11, b12, b13, b14, b15) \
+    Z4(b0) Z4(b1) Z4(b2) Z4(b3) Z4(b4) Z4(b5) Z4(b6) Z4(b7) Z4(b8) Z4(b9) Z4(b10) Z4(b11) Z4(b12) Z4(b13) Z4(b14) Z4(b15)
+    asm volatile(Z16(0, 1, 2, 3, 4, 5, 6, 7, 8, 9, 10, 11, 12, 13, 14, 15) Z16(16, 17, 18, 19, 20, 21, 22, 23, 24, 25, 26, 27, 28, 29, 30, 31)
+                 Z16(32, 33, 34, 35, 36, 37, 38, 39, 40, 41, 42, 43, 44, 45, 46, 47) Z16(48, 49, 50, 51, 52, 53, 54, 55, 56, 57, 58, 59, 60, 61, 62, 63)
+                 :
+                 :
+                 : "a0", "a1", "a2", "a3", "a4", "a5", "a6", "a7", "a8", "a9", "a10", "a11", "a12", "a13", "a14", "a15", "a16", "a17", "a18", "a19",
+                   "a20", "a21", "a22", "a23", "a24", "a25", "a26", "a27", "a28", "a29", "a30", "a31", "a32", "a33", "a34", "a35", "a36", "a37",
+                   "a38", "a39", "a40", "a41", "a42", "a43", "a44", "a45", "a46", "a47", "a48", "a49", "a50", "a51", "a52", "a53", "a54", "a55",
+                   "a56", "a57", "a58", "a59", "a60", "a61", "a62", "a63");
+    asm volatile(Z16(64, 65, 66, 67, 68, 69, 70, 71, 72, 73, 74, 75, 76, 77, 78, 79) Z16(80, 81, 82, 83, 84, 85, 86, 87, 88, 89, 90, 91, 92, 93, 94, 95)
+                 Z16(96, 97, 98, 99, 100, 101, 102, 103, 104, 105, 106, 107, 108, 109, 110, 111)
+                 Z16(112, 113, 114, 115, 116, 117, 118, 119, 120, 121, 122, 123, 124, 125, 126, 127)
+                 :
+                 :
+                 : "a64", "a65", "a66", "a67", "a68", "a69", "a70", "a71", "a72", "a73", "a74", "a75", "a76", "a77", "a78", "a79", "a80", "a81",
+                   "a82", "a83", "a84", "a85", "a86", "a87", "a88", "a89", "a90", "a91", "a92", "a93", "a94", "a95", "a96", "a97", "a98", "a99",
+                   "a100", "a101", "a102", "a103", "a104", "a105", "a106", "a107", "a108", "a109", "a110", "a111", "a112", "a113", "a114",
+                   "a115", "a116", "a117", "a118", "a119", "a120", "a121", "a122", "a123", "a124", "a125", "a126", "a127");
+#undef Z16
+#undef Z4
+}
+
+// The four MFMAs of one op on block row R of the wavefront: a[16R + 4t .. + 3] += b[t] x a.
+template <int R>
+__device__ __forceinline__ void mfma_row(const f16x8 (&b)[TN], const f16x8 &a)
+{
+    asm volatile("s_nop 1\n\t"
+                 "v_mfma_f32_16x16x32_f16 a[%5:%6], %0, %4, a[%5:%6]\n\t"
+                 "v_mfma_f32_16x16x32_f16 a[%7:%8], %1, %4, a[%7:%8]\n\t"
+                 "v_mfma_f32_16x16x32_f16 a[%9:%10], %2, %4, a[%9:%10]\n\t"
+                 "v_mfma_f32_16x16x32_f16 a[%11:%12], %3, %4, a[%11:%12]"
+                 :
+                 : "v"(b[0]), "v"(b[1]), "v"(b[2]), "v"(b[3]), "v"(a), "n"(16 * R), "n"(16 * R + 3), "n"(16 * R + 4), "n"(16 * R + 7),
+                   "n"(16 * R + 8), "n"(16 * R + 11), "n"(16 * R + 12), "n"(16 * R + 15));
+}
+
+// Reads accumulator tile (R, T) after the last MFMA has retired.
+template <int R, int T>
+__device__ __forceinline__ f32x4 read_acc()
+{
+    f32x4 v;
+    asm volatile("v_accvgpr_read_b32 %0, a[%4]\n\tv_accvgpr_read_b32 %1, a[%5]\n\tv_accvgpr_read_b32 %2, a[%6]\n\tv_accvgpr_read_b32 %3, a[%7]"
+                 : "=v"(v[0]), "=v"(v[1]), "=v"(v[2]), "=v"(v[3])
+                 : "n"(16 * R + 4 * T), "n"(16 * R + 4 * T + 1), "n"(16 * R + 4 * T + 2), "n"(16 * R + 4 * T + 3));
+    return v;
 }
 
 } // namespace
-
-typedef uint32_t u32x16 __attribute__((ext_vector_type(16)));
-
-// The op table of (record, wavefront): 8 slots of {w0, w1}.  Read through the constant
-// address space with a wave-uniform address: one scalar load, no vector memory
-// instruction and no v_readlane to get at a slot.
-__device__ __forceinline__ u32x16 load_op_table(const SweepOp *__restrict__ ops, int record, int wave)
-{
-    static_assert(SWEEP_CAP * sizeof(SweepOp) == sizeof(u32x16), "one table = 16 dwords");
-    typedef const __attribute__((address_space(4))) u32x16 *table_ptr;
-    return *(table_ptr)(uintptr_t)(ops + ((long)record * W + wave) * SWEEP_CAP);
-}
-
-// LDS byte offset (without the per-lane XOR) of a slab of the staged chunk
-__device__ __forceinline__ uint32_t slab_offset(uint32_t slab)
-{
-    return (slab >> 3) * (uint32_t)(NT * 256) + (slab & 7u) * 32u;
-}
 
 template <bool C_F32>
 __global__ __launch_bounds__(THREADS) void spmm_sweep_kernel(
     const uint16_t *__restrict__ vals, const uint16_t *__restrict__ B, void *__restrict__ Cout,
     const int32_t *__restrict__ rg_chunk_ptr, const int32_t *__restrict__ chunk_ids,
-    const SweepOp *__restrict__ ops, int Mb, int N, long K, int n_rg, int n_panels)
+    const int32_t *__restrict__ op_ptr, const SweepOp *__restrict__ ops, int Mb, int N, long K, int n_rg, int n_panels,
+    uint32_t vals_bytes)
 {
     extern __shared__ __align__(16) unsigned char lds[];
-    constexpr int CAP = SWEEP_CAP;
 
     const int tid = threadIdx.x;
     const int lane = tid & 63;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
 
-    // panel-major work order, row group fastest; each XCD gets a contiguous eighth
+    // Tile order: blocks of 4 row groups; inside a block panel-major, row group fastest.  Each XCD
+    // (workgroup id modulo 8) takes a contiguous eighth, so the 32 workgroups it runs at a time are
+    // 4 row groups x 8 panels: every A block is wanted by 8 of them, every B chunk by 4.
     const int total = n_rg * n_panels;
     const int per_xcd = gridDim.x >> 3;
-    const int wg = (blockIdx.x & 7) * per_xcd + (blockIdx.x >> 3);
-    if (wg >= total) return;
-    const int panel = wg / n_rg;
-    const int rg = wg - panel * n_rg;
+    const int tile = (blockIdx.x & 7) * per_xcd + (blockIdx.x >> 3);
+    if (tile >= total) return;
+    constexpr int RGB = 4;
+    const int n_blk = (n_rg + RGB - 1) / RGB;
+    int gb = tile / (RGB * n_panels);
+    gb = gb < n_blk - 1 ? gb : n_blk - 1;
+    const int rem = tile - gb * RGB * n_panels;
+    const int rgs_here = n_rg - gb * RGB < RGB ? n_rg - gb * RGB : RGB;
+    const int panel = rem / rgs_here;
+    const int rg = gb * RGB + rem - panel * rgs_here;
     const int n0 = panel * NT;
 
     const int i16 = lane & 15, g = lane >> 4, sel = g >> 1, kh = g & 1;
-    // column (within the panel) of MFMA row i16 in tile 0; tile t adds 64*(t/4) + 4*(t%4).
+    const uint32_t lbase = (uint32_t)(uintptr_t)(__attribute__((address_space(3))) void *)lds;
+    // column (within the panel) of MFMA row i16 in n-tile 0 is 16*(i16>>2) + (i16&3); n-tile t adds 4*t.
     // The swizzle value of every such column equals i16.
-    const int n_lane = 16 * (i16 >> 2) + (i16 & 3);
-    const int rd_base = n_lane * ROW_BYTES;
+    const uint32_t rd_lane = (uint32_t)(16 * (i16 >> 2) + (i16 & 3)) * ROW_BYTES; // byte offset in a stage
     const uint32_t lane_xor = (uint32_t)((kh ^ i16) << 4); // ((2*slab | kh) ^ i16) << 4 == (slab * 32) ^ lane_xor
-
-    f32x4 acc[RW][TN];
-#pragma unroll
-    for (int r = 0; r < RW; r++)
-#pragma unroll
-        for (int t = 0; t < TN; t++) acc[r][t] = (f32x4){0.f, 0.f, 0.f, 0.f};
-
-    const int c_begin = rg_chunk_ptr[rg], c_end = rg_chunk_ptr[rg + 1];
     const uint32_t a_lane_bytes = (uint32_t)(i16 * 16 + kh * 8) * 2u; // this lane's 16 bytes inside a block
-    const f16x8 zero8 = {0, 0, 0, 0, 0, 0, 0, 0};
 
-    // A operands of one chunk: slot k <- the two blocks of op k (lanes 0-31: first block,
-    // 32-63: second).  Empty slots load nothing: a vector memory instruction costs the
-    // load path of the CU 16 clocks whatever it fetches.  The missing second block of a
-    // single re-reads the first (zeroed at use).
-    auto load_a = [&](f16x8 (&dst)[CAP], const u32x16 &tab) {
-        constexpr int CAPR = CAP / RW;
+    // The 8 x 4 accumulator tiles (4 registers each) live in a[0:127], tile (r, t) in a[16r + 4t .. + 3], and are
+    // touched only by the assembly below: which block row an op adds to is known at run time only, and a
+    // run-time choice between register sets is a branch between otherwise identical MFMA groups.
+    zero_accumulators();
+
+    // vals as a raw buffer: base, no stride, nnzb * 512 bytes, 32-bit untyped data
+    i32x4 vals_rsrc;
+    vals_rsrc[0] = (int)(uint32_t)(uintptr_t)vals;
+    vals_rsrc[1] = (int)(uint32_t)((uintptr_t)vals >> 32) & 0xffff;
+    vals_rsrc[2] = (int)vals_bytes;
+    vals_rsrc[3] = 0x00020000;
+
+    const int c_begin = rg_chunk_ptr[rg], n_chunks = rg_chunk_ptr[rg + 1] - c_begin;
+    const int op_begin = op_ptr[rg * W + wave];
+    const int n_ops = op_ptr[rg * W + wave + 1] - op_begin;
+
+    if (n_chunks > 0) { // uniform over the workgroup: every wavefront has the chunk list of its row group
+        // Vector memory instructions complete in order.  `age` counts the ops (= A loads) since the last chunk
+        // boundary, `burst` the copy instructions issued at that boundary: together they give the immediate of
+        // every vmcnt wait.
+        int age = 0, burst = 0;
+        auto lds_copy = [&](uint32_t voff, const void *sbase, uint32_t dst) { // 64 lanes x 16 B -> LDS dst + lane * 16
+            asm volatile("s_mov_b32 m0, %2\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, %1"
+                         :
+                         : "v"(voff), "s"(sbase), "s"(dst)
+                         : "memory");
+            burst++;
+        };
+
+        // ---- B panel copies: this wavefront fills rows ((wave & 3) * 4 + it) * 4 .. + 3 of slab group wave / 4 ----
+        // lane -> (row q = lane / 16, physical slot ps = lane % 16); logical slot = ps ^ swizzle(n),
+        // swizzle(n) = (n & 3) | ((n >> 2) & 12) = q | (wave & 3) << 2 for these rows.
+        const int q = lane >> 4;
+        const uint32_t ls = (uint32_t)((lane & 15) ^ (q | ((wave & 3) << 2)));
+        const uint32_t k_lane = (uint32_t)(wave >> 2) * 128u + ls * 8u; // k inside the chunk
+        const uint32_t col_lane = (uint32_t)q * (uint32_t)K;            // elements; the launcher checks K < 2^28
+        const uint32_t kmax = (uint32_t)K - 8u;
+        auto issue_copies = [&](int cl) {
+            const uint32_t k0 = (uint32_t)chunk_ids[c_begin + cl] * (uint32_t)(S * 16);
+            uint32_t k = k0 + k_lane;
+            k = k < kmax ? k : kmax; // slabs past K are referenced by no op; keep the read inside the matrix
+            const uint32_t voff = (col_lane + k) * 2u;
+            const uint32_t dst0 = lbase + (uint32_t)(cl % NS) * STAGE_BYTES + (uint32_t)(wave * COPIES) * 1024u;
 #pragma unroll
-        for (int r = 0; r < RW; r++) {
-#pragma unroll
-            for (int j = 0; j < CAPR; j++) {
-                const int k = r * CAPR + j;
-                const uint32_t w0 = tab[2 * k], w1 = tab[2 * k + 1];
-                if (w0 == SWEEP_EMPTY_SLOT) break; // the slots of a block row fill up in order
-                const uint32_t b1 = (w0 & 0xFFFFFFu) * 512u; // nnzb < 2^23 is checked by the plan
-                const uint32_t p2 = w1 & 0xFFFFFFu;
-                const uint32_t b2 = p2 == SWEEP_NO_BLOCK ? b1 : p2 * 512u;
-                const uint32_t off = (sel ? b2 : b1) + a_lane_bytes;
-                dst[k] = *reinterpret_cast<const f16x8 *>(reinterpret_cast<const char *>(vals) + off);
+            for (int it = 0; it < COPIES; it++) {
+                const int row4 = ((wave & 3) * 4 + it) * 4; // first of four columns, wave-uniform
+                if (n0 + row4 >= N) continue;               // N % 8 == 0: all four columns or none
+                lds_copy(voff, B + (long)(n0 + row4) * K, dst0 + (uint32_t)it * 1024u);
             }
-        }
-    };
+        };
 
-    // Two sets of op-table registers and of A operand registers; consecutive records use
-    // them in swapped roles (the loop below is unrolled by two), so nothing is copied.
-    u32x16 tab0, tab1;
-#pragma unroll
-    for (int k = 0; k < 16; k++) { tab0[k] = SWEEP_EMPTY_SLOT; tab1[k] = SWEEP_EMPTY_SLOT; }
-    f16x8 a0[CAP], a1[CAP];
-#pragma unroll
-    for (int k = 0; k < CAP; k++) { a0[k] = zero8; a1[k] = zero8; }
+        // ---- op descriptors: windows of 64 ops (1 KiB, one copy instruction) in three LDS slots per wavefront ----
+        const SweepOp *op_base = ops + op_begin; // the plan pads the array: reads past n_ops stay inside it
+        const uint32_t win_base = (uint32_t)(NS * STAGE_BYTES) + (uint32_t)wave * (WIN_SLOTS * 1024u); // byte offset in LDS
+        int win_next = 0; // first window not requested yet
+        auto copy_window = [&]() {
+            lds_copy((uint32_t)lane * 16u, op_base + (long)win_next * 64, lbase + win_base + (uint32_t)(win_next % WIN_SLOTS) * 1024u);
+            win_next++;
+        };
+        // plain LDS read, same address in every lane; made scalar where it is used, several ops later
+        auto read_desc = [&](int x) {
+            return *reinterpret_cast<const uint4 *>(lds + win_base + (uint32_t)((x >> 6) % WIN_SLOTS) * 1024u + (uint32_t)(x & 63) * 16u);
+        };
 
-    int stage = 0;
-    const int last = c_end - 1;
-    if (c_begin < c_end) {
-        tab0 = load_op_table(ops, c_begin, wave);
-        tab1 = load_op_table(ops, c_begin + 1 < last ? c_begin + 1 : last, wave);
-        fill_issue(lds, B, chunk_ids[c_begin] & ~SWEEP_CONT_FLAG, n0, N, K, wave, lane);
-        load_a(a0, tab0);
-    }
-    __builtin_amdgcn_s_waitcnt(0x0f70); // vmcnt(0): the copies of this wavefront have landed
-    __syncthreads();
+        // ---- operand registers ----
+        f16x8 bq[PB + 1][TN];
+        f16x8 aq[DA];
+        uint4 dq[DQ];      // descriptors of ops i .. i + DQ - 1 (slot = op % DQ), one copy per lane
+        uint32_t fq[PB + 1]; // flags and block row (word 1) of the ops whose B operands are under way
+        const f16x8 zero8 = {0, 0, 0, 0, 0, 0, 0, 0};
+        // A operand: one buffer load of the 1 KiB pair, lanes 32-63 take the second block.  Where a block does not
+        // belong to the op its lanes get an offset past the end of the buffer, for which the load returns zeros:
+        // between the load and the MFMAs nothing touches the operand registers.
+        const uint32_t a_voff = (uint32_t)sel * 512u + a_lane_bytes;
+        const uint32_t a_voff_zero_hi = sel ? 0x80000000u : a_voff;
+        const uint32_t a_voff_zero_lo = sel ? a_voff : 0x80000000u;
+        const uint32_t a_voff_zero = 0x80000000u;
 
-    // One record: tab_c / a_c hold the op table and A operands of record ci, tab_n the table of
-    // record ci + 1, whose A operands go to a_n.
-    auto record = [&](int ci, u32x16 &tab_c, const u32x16 &tab_n, f16x8 (&a_c)[CAP], f16x8 (&a_n)[CAP]) {
-        // ---- everything record ci+1 needs ----
-        bool next_is_new = false;
-        if (ci + 1 < c_end) {
-            load_a(a_n, tab_n);
-            // A record that continues the chunk of the previous record (its ops did not
-            // fit one table) has bit 30 set: no B copy, the LDS stage stays.
-            const int next_chunk = chunk_ids[ci + 1];
-            next_is_new = !(next_chunk & SWEEP_CONT_FLAG);
-            if (next_is_new)
-                fill_issue(lds + (stage ^ 1) * STAGE_BYTES, B, next_chunk, n0, N, K, wave, lane);
-        }
-        // ---- MFMA work of record ci: registers and LDS only ----
-        const unsigned char *cur = lds + stage * STAGE_BYTES + rd_base;
+        // reads the B operands of an op: lanes 0-31 from the slab of its first block, 32-63 of the second
+        auto issue_b = [&](f16x8(&b)[TN], uint32_t w1, uint32_t w2) {
+            const uint32_t off0 = w1 & SWEEP_LDS_MASK, off1 = w2;
+            const unsigned char *p = lds + rd_lane + ((sel ? off1 : off0) ^ lane_xor);
 #pragma unroll
-        for (int r = 0; r < RW; r++) {
-            // table slot k belongs to block row k / CAPR of this wavefront: the accumulator
-            // registers of every slot are fixed at compile time
-            constexpr int CAPR = CAP / RW;
-#pragma unroll
-            for (int j = 0; j < CAPR; j++) {
-                const int k = r * CAPR + j;
-                const uint32_t w0 = tab_c[2 * k], w1 = tab_c[2 * k + 1];
-                if (w0 == SWEEP_EMPTY_SLOT) break; // the slots of a block row fill up in order
-                const uint32_t soff = sel ? slab_offset(w1 >> 24) : slab_offset(w0 >> 24);
-                const unsigned char *bp = cur + (soff ^ lane_xor);
-                f16x8 av = a_c[k];
-                if ((w1 & 0xFFFFFFu) == SWEEP_NO_BLOCK) // single: no second block
-                    av = sel ? zero8 : av;
-#pragma unroll
-                for (int u = 0; u < TN / 4; u++) {
-                    f16x8 b[4];
-#pragma unroll
-                    for (int tt = 0; tt < 4; tt++)
-                        b[tt] = *reinterpret_cast<const f16x8 *>(bp + (64 * u + 4 * tt) * ROW_BYTES);
-#pragma unroll
-                    for (int tt = 0; tt < 4; tt++)
-                        acc[r][u * 4 + tt] = __builtin_amdgcn_mfma_f32_16x16x32_f16(
-                            b[tt], av, acc[r][u * 4 + tt], 0, 0, 0);
-                }
-                // order of the 8 LDS reads and 8 MFMAs of this op: four reads ahead, then one
-                // MFMA per further read, so an MFMA never waits on the read issued just before it
-                __builtin_amdgcn_sched_group_barrier(0x100, 4, 0);
-#pragma unroll
-                for (int q = 0; q < 4; q++) {
-                    __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
-                    __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);
-                }
-                __builtin_amdgcn_sched_group_barrier(0x008, 4, 0);
-            }
-        }
-        // the table of record ci+2 replaces the one just used (a scalar load: it returns
-        // while this wavefront waits for the copies and at the barrier)
-        if (ci + 2 <= last) tab_c = load_op_table(ops, ci + 2, wave);
-        __builtin_amdgcn_s_waitcnt(0x0f70); // vmcnt(0): next record's B and A have landed
+            for (int tt = 0; tt < TN; tt++) b[tt] = *reinterpret_cast<const f16x8 *>(p + tt * 4 * ROW_BYTES);
+        };
+        // loads the A operand of an op: its two blocks are neighbours in vals, 1 KiB in MFMA operand order
+        auto issue_a = [&](f16x8 &a, uint32_t w0, uint32_t w1) {
+            const uint32_t z = w1 & (SWEEP_OP_ZERO_HI | SWEEP_OP_ZERO_LO);
+            if (z == 0)
+                asm volatile("buffer_load_dwordx4 %0, %1, %2, %3 offen" : "=v"(a) : "v"(a_voff), "s"(vals_rsrc), "s"(w0));
+            else if (z == SWEEP_OP_ZERO_HI)
+                asm volatile("buffer_load_dwordx4 %0, %1, %2, %3 offen" : "=v"(a) : "v"(a_voff_zero_hi), "s"(vals_rsrc), "s"(w0));
+            else if (z == SWEEP_OP_ZERO_LO)
+                asm volatile("buffer_load_dwordx4 %0, %1, %2, %3 offen" : "=v"(a) : "v"(a_voff_zero_lo), "s"(vals_rsrc), "s"(w0));
+            else
+                asm volatile("buffer_load_dwordx4 %0, %1, %2, %3 offen" : "=v"(a) : "v"(a_voff_zero), "s"(vals_rsrc), "s"(w0));
+        };
+
+        // ---- prologue: chunks 0 and 1 resident, descriptors of the first 192 ops, first operands under way ----
+        issue_copies(0);
+        if (n_chunks > 1) issue_copies(1);
+        copy_window();
+        copy_window();
+        copy_window();
+        asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
         __syncthreads();
-        if (next_is_new) stage ^= 1;
-    };
-    for (int ci = c_begin; ci < c_end; ci += 2) {
-        record(ci, tab0, tab1, a0, a1);
-        if (ci + 1 < c_end) record(ci + 1, tab1, tab0, a1, a0);
-    }
-    // Epilogue: acc[r][t][e] = C[(rg*G + wave*RW + r)*16 + i16][n0 + 64*(t/4) + 16*g + 4*(t%4) + e]
 #pragma unroll
-    for (int r = 0; r < RW; r++) {
-        const int br = rg * SWEEP_G + wave * RW + r;
-        if (br >= Mb) continue;
-        const long m = (long)br * 16 + i16;
+        for (int d = 0; d < DQ; d++) dq[d] = read_desc(d);
 #pragma unroll
-        for (int u = 0; u < TN / 4; u++) {
-            const int nbase = n0 + 64 * u + 16 * g;
-            if (C_F32) {
-                float *crow = reinterpret_cast<float *>(Cout) + m * (long)N;
+        for (int d = 0; d < AHEAD; d++)
+            issue_a(aq[d], __builtin_amdgcn_readfirstlane(dq[d].x), __builtin_amdgcn_readfirstlane(dq[d].y));
+        burst = 0;
+        if (n_chunks > 2) issue_copies(2); // after the first A loads, like the copies of a boundary
 #pragma unroll
-                for (int tt = 0; tt < 4; tt++)
-                    if (nbase + 4 * tt < N)
-                        *reinterpret_cast<f32x4 *>(crow + nbase + 4 * tt) = acc[r][u * 4 + tt];
-            } else {
-                uint16_t *crow = reinterpret_cast<uint16_t *>(Cout) + m * (long)N;
+        for (int d = AHEAD; d < DA; d++) aq[d] = zero8;
 #pragma unroll
-                for (int tt = 0; tt < 4; tt += 2) {
-                    const f32x4 v0 = acc[r][u * 4 + tt], v1 = acc[r][u * 4 + tt + 1];
-                    f16x8 h = {(_Float16)v0[0], (_Float16)v0[1], (_Float16)v0[2], (_Float16)v0[3],
-                               (_Float16)v1[0], (_Float16)v1[1], (_Float16)v1[2], (_Float16)v1[3]};
-                    if (nbase + 4 * tt < N) *reinterpret_cast<f16x8 *>(crow + nbase + 4 * tt) = h;
-                }
-            }
+        for (int d = 0; d < PB; d++) {
+            fq[d] = __builtin_amdgcn_readfirstlane(dq[d].y);
+            issue_b(bq[d], fq[d], __builtin_amdgcn_readfirstlane(dq[d].z));
         }
+        fq[PB] = 0;
+#pragma unroll
+        for (int tt = 0; tt < TN; tt++) bq[PB][tt] = zero8;
+
+        int cur = 0; // chunk (index into the row group's chunk list) the executed ops belong to
+        int i = 0;   // op executed next
+
+        // One op.  J = i % UNROLL selects the register sets.
+        auto step = [&](auto jc) {
+            constexpr int J = decltype(jc)::value;
+            const uint32_t w1 = fq[J % (PB + 1)];
+            if (w1 & SWEEP_OP_BOUNDARY) {
+                // entering chunk cur: the copies of chunk cur + 1 (issued when chunk cur - 1 was entered, `age` A
+                // loads ago) have landed; after the barrier every wavefront is done with chunk cur - 1, and the
+                // stage of chunk cur - 2 takes the copies of chunk cur + 2
+                cur++;
+                if (age <= AHEAD) { // else an A load issued after them has been waited for
+                    if (age == 2) asm volatile("s_waitcnt vmcnt(2)" ::: "memory");
+                    else if (age == 3) asm volatile("s_waitcnt vmcnt(3)" ::: "memory");
+                    else if (age == 4) asm volatile("s_waitcnt vmcnt(4)" ::: "memory");
+                    else asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+                }
+                asm volatile("s_barrier" ::: "memory");
+                burst = 0;
+                age = 0;
+                if (cur + 2 < n_chunks) issue_copies(cur + 2);
+                // descriptor windows: those up to two ahead of the current op are requested here; a chunk holds
+                // at most 72 ops of a wavefront, so a window is requested at least 50 ops before its first read
+                // and the windows requested at the last boundary cover the read-ahead past the last op
+                while ((i >> 6) + 2 >= win_next) copy_window();
+            }
+            // Operands of later ops.  Unconditional: past the end of the stream the descriptors are the plan's
+            // padding (block 0, first slab), whose operands are fetched and never used.  A condition here would
+            // make the compiler wait for every LDS read before the MFMAs (it has to assume the path on which
+            // the younger reads were not issued).
+            {
+                const uint4 &db = dq[(J + PB) % DQ];
+                fq[(J + PB) % (PB + 1)] = __builtin_amdgcn_readfirstlane(db.y);
+                issue_b(bq[(J + PB) % (PB + 1)], fq[(J + PB) % (PB + 1)], __builtin_amdgcn_readfirstlane(db.z));
+                const uint4 &da = dq[(J + AHEAD) % DQ];
+                issue_a(aq[(J + AHEAD) % DA], __builtin_amdgcn_readfirstlane(da.x), __builtin_amdgcn_readfirstlane(da.y));
+                dq[J % DQ] = read_desc(i + DQ); // replaces the descriptor of op i, whose word 1 is in w1
+            }
+            __builtin_amdgcn_sched_barrier(0);
+            // the A operand of op i: AHEAD younger A loads, and the copies of the last boundary if that young
+            // (the waits carry no operands: an operand tied to the wait lets the compiler copy the register
+            // before it; the operand registers go from the load straight to the MFMAs)
+            if (age < AHEAD) {
+                if (burst == COPIES) asm volatile("s_waitcnt vmcnt(8)" ::: "memory");
+                else if (burst == COPIES + 1) asm volatile("s_waitcnt vmcnt(9)" ::: "memory");
+                else if (burst == COPIES + 2) asm volatile("s_waitcnt vmcnt(10)" ::: "memory");
+                else asm volatile("s_waitcnt vmcnt(4)" ::: "memory"); // fewer copies (last panel, last chunks): waits for them too
+            } else {
+                asm volatile("s_waitcnt vmcnt(4)" ::: "memory");
+            }
+            static_assert(AHEAD == 4 && COPIES == 4, "immediates above");
+            age++;
+            const f16x8 &av = aq[J % DA];
+            f16x8(&bc)[TN] = bq[J % (PB + 1)];
+            switch (w1 >> 28) {
+            case 0: mfma_row<0>(bc, av); break;
+            case 1: mfma_row<1>(bc, av); break;
+            case 2: mfma_row<2>(bc, av); break;
+            case 3: mfma_row<3>(bc, av); break;
+            case 4: mfma_row<4>(bc, av); break;
+            case 5: mfma_row<5>(bc, av); break;
+            case 6: mfma_row<6>(bc, av); break;
+            default: mfma_row<7>(bc, av); break;
+            }
+        };
+        while (i < n_ops) {
+            step(std::integral_constant<int, 0>{}); if (++i >= n_ops) break;
+            step(std::integral_constant<int, 1>{}); if (++i >= n_ops) break;
+            step(std::integral_constant<int, 2>{}); if (++i >= n_ops) break;
+            step(std::integral_constant<int, 3>{}); if (++i >= n_ops) break;
+            step(std::integral_constant<int, 4>{}); if (++i >= n_ops) break;
+            step(std::integral_constant<int, 5>{}); ++i;
+        }
+        asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
     }
+    asm volatile("s_nop 15\n\ts_nop 15" ::: "memory"); // the last MFMAs retire before their results are read
+
+    // Epilogue: tile (r, t), element e = C[(rg*64 + wave*8 + r)*16 + i16][n0 + 16*g + 4*t + e]
+    auto store_row = [&](auto rc) {
+        constexpr int R = decltype(rc)::value;
+        const int br = rg * SWEEP_G + wave * RW + R;
+        if (br >= Mb) return;
+        const long m = (long)br * 16 + i16;
+        const int nbase = n0 + 16 * g;
+        const f32x4 v0 = read_acc<R, 0>(), v1 = read_acc<R, 1>(), v2 = read_acc<R, 2>(), v3 = read_acc<R, 3>();
+        if (C_F32) {
+            float *crow = reinterpret_cast<float *>(Cout) + m * (long)N + nbase;
+            if (nbase < N) { *reinterpret_cast<f32x4 *>(crow) = v0; *reinterpret_cast<f32x4 *>(crow + 4) = v1; }
+            if (nbase + 8 < N) { *reinterpret_cast<f32x4 *>(crow + 8) = v2; *reinterpret_cast<f32x4 *>(crow + 12) = v3; }
+        } else {
+            uint16_t *crow = reinterpret_cast<uint16_t *>(Cout) + m * (long)N + nbase;
+            const f16x8 h0 = {(_Float16)v0[0], (_Float16)v0[1], (_Float16)v0[2], (_Float16)v0[3],
+                              (_Float16)v1[0], (_Float16)v1[1], (_Float16)v1[2], (_Float16)v1[3]};
+            const f16x8 h1 = {(_Float16)v2[0], (_Float16)v2[1], (_Float16)v2[2], (_Float16)v2[3],
+                              (_Float16)v3[0], (_Float16)v3[1], (_Float16)v3[2], (_Float16)v3[3]};
+            if (nbase < N) *reinterpret_cast<f16x8 *>(crow) = h0;
+            if (nbase + 8 < N) *reinterpret_cast<f16x8 *>(crow + 8) = h1;
+        }
+    };
+    store_row(std::integral_constant<int, 0>{}); store_row(std::integral_constant<int, 1>{});
+    store_row(std::integral_constant<int, 2>{}); store_row(std::integral_constant<int, 3>{});
+    store_row(std::integral_constant<int, 4>{}); store_row(std::integral_constant<int, 5>{});
+    store_row(std::integral_constant<int, 6>{}); store_row(std::integral_constant<int, 7>{});
 }
 
 hipError_t launch_sweep(const SweepArgs &a, hipStream_t st)
 {
-    static bool attr_set[2] = {false, false};
-    const int lds_bytes = 2 * STAGE_BYTES;
-    const int which = a.c_f32 ? 1 : 0;
-    if (!attr_set[which]) {
-        hipError_t e = a.c_f32
-            ? hipFuncSetAttribute(reinterpret_cast<const void *>(&spmm_sweep_kernel<true>),
-                                  hipFuncAttributeMaxDynamicSharedMemorySize, lds_bytes)
-            : hipFuncSetAttribute(reinterpret_cast<const void *>(&spmm_sweep_kernel<false>),
-                                  hipFuncAttributeMaxDynamicSharedMemorySize, lds_bytes);
-        if (e != hipSuccess) return e;
-        attr_set[which] = true;
-    }
+    const int lds_bytes = NS * STAGE_BYTES + WINDOW_BYTES;
+    // dynamic LDS above 64 KiB has to be allowed once per kernel and device; the call is cheap and idempotent
+    hipError_t e = a.c_f32
+        ? hipFuncSetAttribute(reinterpret_cast<const void *>(&spmm_sweep_kernel<true>),
+                              hipFuncAttributeMaxDynamicSharedMemorySize, lds_bytes)
+        : hipFuncSetAttribute(reinterpret_cast<const void *>(&spmm_sweep_kernel<false>),
+                              hipFuncAttributeMaxDynamicSharedMemorySize, lds_bytes);
+    if (e != hipSuccess) return e;
+    if (a.K >= ((size_t)1 << 28)) return hipErrorInvalidValue; // copy offsets: (3 * K + k) * 2 in 32 bits
     const int n_panels = (int)((a.N + NT - 1) / NT);
     long wgs = (long)a.n_rg * n_panels;
     wgs = (wgs + 7) / 8 * 8;
@@ -316,14 +405,13 @@ hipError_t launch_sweep(const SweepArgs &a, hipStream_t st)
     dim3 grid((unsigned)wgs), block(THREADS);
     if (a.c_f32)
         hipLaunchKernelGGL((spmm_sweep_kernel<true>), grid, block, lds_bytes, st, a.vals, a.B, a.C,
-                           a.rg_chunk_ptr, a.chunk_ids, a.ops, (int)(a.M / 16), (int)a.N, (long)a.K,
-                           a.n_rg, n_panels);
+                           a.rg_chunk_ptr, a.chunk_ids, a.op_ptr, a.ops, (int)(a.M / 16), (int)a.N, (long)a.K,
+                           a.n_rg, n_panels, (uint32_t)(a.nnzb * 512));
     else
         hipLaunchKernelGGL((spmm_sweep_kernel<false>), grid, block, lds_bytes, st, a.vals, a.B, a.C,
-                           a.rg_chunk_ptr, a.chunk_ids, a.ops, (int)(a.M / 16), (int)a.N, (long)a.K,
-                           a.n_rg, n_panels);
+                           a.rg_chunk_ptr, a.chunk_ids, a.op_ptr, a.ops, (int)(a.M / 16), (int)a.N, (long)a.K,
+                           a.n_rg, n_panels, (uint32_t)(a.nnzb * 512));
     return hipGetLastError();
 }
 
 } // namespace smat
-

@@ -1,0 +1,28 @@
+// Host-side work list of the sweep kernel (see spmm_sweep.hip): per row group of 64 block rows the
+// K chunks it touches, per (row group, wavefront) a stream of ops.  Plain C++: built and checked
+// without a GPU.
+#pragma once
+#include <stddef.h>
+#include <stdint.h>
+
+#include <vector>
+
+namespace smat {
+
+struct SweepOpHost { // layout: SweepOp in spmm_kernels.h
+    uint32_t w0, w1, w2, w3;
+};
+
+struct SweepPlanHost {
+    std::vector<int32_t> rg_chunk_ptr; // n_rg + 1
+    std::vector<int32_t> chunk_ids;    // K chunk of every (row group, listed chunk)
+    std::vector<int32_t> op_ptr;       // n_rg * 8 + 1
+    std::vector<SweepOpHost> ops;      // op streams + padding
+    size_t n_pairs = 0, n_singles = 0, n_fillers = 0;
+};
+
+// row_ptr / col_idx: host BCSR (col_idx = absolute first column of each block, validated by the caller);
+// at least two blocks.
+void build_sweep_plan(const int32_t *row_ptr, const int32_t *col_idx, size_t mb, size_t kb, SweepPlanHost &out);
+
+} // namespace smat

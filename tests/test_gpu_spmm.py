@@ -191,10 +191,12 @@ SWEEP = 2
     (9, 13, 0.35, 128),     # fewer block rows than one row group, one partial K chunk
     (40, 40, 0.15, 136),    # partial last panel, partial last row group
     (64, 33, 0.10, 256),    # K = 528: last chunk is 1 slab wide
-    (33, 70, 0.05, 520),    # sparse enough that some (row group, chunk) records are empty
+    (33, 70, 0.05, 520),    # sparse enough that wavefronts get filler ops and blocks pair across chunks
     (32, 16, 1.00, 128),    # fully dense: every op is a pair
     (35, 3, 0.60, 8),       # narrowest N, K = 48: one partial chunk, most of the panel unused
-    (70, 20, 0.30, 72),     # N below one panel
+    (70, 20, 0.30, 72),     # N just above one panel
+    (130, 160, 1.00, 64),   # dense, ten chunks: 64 ops per wavefront and chunk, several descriptor windows
+    (200, 300, 0.12, 192),  # four row groups, 19 chunks: the ring of stages wraps several times
 ])
 def test_sweep_kernel_matches_oracle(smat, cuda, oracle, mb, kb, density, N):
     A = gen.random_bcsr(mb, kb, density, seed=1000 + mb + kb)
@@ -224,17 +226,22 @@ def test_sweep_needs_a_plan_with_col_idx(smat, cuda):
         smat.Plan(A["b_row_ptr"], A["M"], A["K"], A["nnzb"], 128, col_idx_host=None, kernel=SWEEP)
 
 
-def test_sweep_refuses_a_b_of_4_gib_or_more(smat, cuda):
-    """The sweep kernel addresses B with 32-bit byte offsets: an explicit request is refused before any
-    launch (the buffers here are dummies that are never touched)."""
+def test_sweep_refuses_what_it_cannot_address(smat, cuda):
+    """The sweep kernel addresses blocks in pairs and B with 32-bit offsets inside four columns: a single
+    block is refused when the plan is made, K >= 2^28 at the launch (the buffers here are dummies that are
+    never touched)."""
     import torch
-    M, K, N = 16, 65536, 32768  # K * N * 2 bytes = 4 GiB
     rp = np.array([0, 1], np.int32)
     ci = np.array([0], np.int32)
-    plan = smat.Plan(rp, M, K, 1, 128, col_idx_host=ci, kernel=SWEEP)
+    with pytest.raises(smat.SmatError):
+        smat.Plan(rp, 16, 64, 1, 128, col_idx_host=ci, kernel=SWEEP)
+    M, K, N = 16, 1 << 28, 64
+    rp = np.array([0, 2], np.int32)
+    ci = np.array([0, 16], np.int32)
+    plan = smat.Plan(rp, M, K, 2, 64, col_idx_host=ci, kernel=SWEEP)
     dummy = torch.zeros(4096, dtype=torch.int16, device=cuda)
     with pytest.raises(smat.SmatError):
-        smat.spmm(dummy, to_dev(torch, rp, cuda), to_dev(torch, ci, cuda), dummy, dummy, M, N, K, 1, plan=plan, kernel=SWEEP)
+        smat.spmm(dummy, to_dev(torch, rp, cuda), to_dev(torch, ci, cuda), dummy, dummy, M, N, K, 2, plan=plan, kernel=SWEEP)
     plan.close()
 
 
@@ -286,7 +293,7 @@ def test_config5_stencil_reduced_and_reordered(smat, cuda, oracle):
 
 def test_plan_takes_the_sweep_kernel_only_when_it_fills_the_device(smat, cuda, oracle):
     import torch
-    # 64 groups of 32 block rows, 10 % of the blocks: 4 panels of 128 columns make 256 workgroups
+    # 32 groups of 64 block rows, 10 % of the blocks: 8 panels of 64 columns make 256 workgroups
     A = gen.random_bcsr(2048, 32, 0.10, seed=77)
     M, K, nnzb = A["M"], A["K"], A["nnzb"]
     wide = smat.Plan(A["b_row_ptr"], M, K, nnzb, 512, col_idx_host=A["b_col_idx"])

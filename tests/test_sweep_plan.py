@@ -1,0 +1,160 @@
+"""Work list of the sweep kernel, checked on the CPU: the op streams are replayed in numpy with the
+kernel's own rules (which LDS stages are resident when an op runs, at least two ops per wavefront and
+chunk, one barrier per chunk boundary in every wavefront) and the replay has to give A x B.
+
+What the replay pins: every block is multiplied exactly once, with the rows of B under its block
+column, into its own block row; the stage an op reads holds the chunk it needs at that moment."""
+import ctypes as C
+
+import numpy as np
+import pytest
+
+from smat_amd import generators as gen
+from smat_amd._lib import lib
+
+G, RW, WAVES, S, STAGES = 64, 8, 8, 16, 4
+ZERO_HI, ZERO_LO, BOUNDARY = 1, 2, 4
+LDS_MASK = 0x1C0E0
+PAD = 384
+
+
+def sweep_plan(row_ptr, col_idx, M, K):
+    fn = lib.smat_internal_sweep_plan
+    fn.restype = C.c_int
+    fn.argtypes = [C.c_void_p, C.c_void_p, C.c_size_t, C.c_size_t] + [C.POINTER(C.c_void_p)] * 4 + [C.POINTER(C.c_int64)]
+    row_ptr = np.ascontiguousarray(row_ptr, np.int32)
+    col_idx = np.ascontiguousarray(col_idx, np.int32)
+    out = [C.c_void_p() for _ in range(4)]
+    counts = (C.c_int64 * 6)()
+    rc = fn(row_ptr.ctypes.data, col_idx.ctypes.data, M, K, *[C.byref(o) for o in out], counts)
+    assert rc == 0
+    n_rg, n_chunks, n_ops = counts[0], counts[1], counts[2]
+
+    def take(ptr, n, dtype):
+        a = np.ctypeslib.as_array(C.cast(ptr, C.POINTER(np.ctypeslib.as_ctypes_type(dtype))), shape=(n,)).copy()
+        lib.smat_host_free(ptr)
+        return a
+    return {
+        "rg_chunk_ptr": take(out[0], n_rg + 1, np.int32), "chunk_ids": take(out[1], n_chunks, np.int32),
+        "op_ptr": take(out[2], n_rg * WAVES + 1, np.int32), "ops": take(out[3], (n_ops + PAD) * 4, np.uint32).reshape(-1, 4),
+        "pairs": counts[3], "singles": counts[4], "fillers": counts[5], "n_ops": n_ops,
+    }
+
+
+def slot_of(off):
+    """LDS offset -> (stage, block column inside the chunk)"""
+    assert off & ~LDS_MASK == 0
+    slot = (off >> 14) * 8 + ((off >> 5) & 7)
+    return slot // S, slot % S
+
+
+def replay(plan, A, Bd):
+    """Runs the op streams on dense numpy operands. A: dict from gen (BCSR), Bd: K x N float64."""
+    M, K, rp, ci = A["M"], A["K"], A["b_row_ptr"], A["b_col_idx"]
+    blocks = A["b_val"].view(np.float16).astype(np.float64).reshape(-1, 16, 16)
+    nnzb = ci.size
+    Cd = np.zeros((M, Bd.shape[1]))
+    used = np.zeros(nnzb, int)
+    block_row = np.repeat(np.arange(M // 16), np.diff(rp))
+    n_rg = plan["rg_chunk_ptr"].size - 1
+    for rg in range(n_rg):
+        chunks = plan["chunk_ids"][plan["rg_chunk_ptr"][rg]:plan["rg_chunk_ptr"][rg + 1]]
+        assert np.all(np.diff(chunks) > 0)
+        for w in range(WAVES):
+            ops = plan["ops"][plan["op_ptr"][rg * WAVES + w]:plan["op_ptr"][rg * WAVES + w + 1]]
+            if chunks.size == 0:
+                assert ops.shape[0] == 0
+                continue
+            cur, in_chunk = 0, 0
+            for w0, w1, w2, w3 in ops:
+                if w1 & BOUNDARY:
+                    assert in_chunk >= 2, "fewer than two ops in a chunk"
+                    cur, in_chunk = cur + 1, 0
+                in_chunk += 1
+                q = int(w0) // 512
+                assert int(w0) % 512 == 0 and 0 <= q and q + 1 < nnzb and w3 == 0
+                r = int(w1) >> 28
+                br = rg * G + w * RW + r
+                for half, (off, zero) in enumerate(((int(w1) & LDS_MASK, w1 & ZERO_LO), (int(w2), w1 & ZERO_HI))):
+                    stage, slab = slot_of(off)
+                    # the stage holds chunk position cur or cur - 1 (whichever maps to it); cur + 1 is also
+                    # resident but no op may use it yet
+                    pos = [p for p in (cur, cur - 1) if p >= 0 and p % STAGES == stage]
+                    assert pos, "op reads a stage that holds neither its chunk nor the previous one"
+                    if zero:
+                        continue
+                    blk = q + half
+                    k0 = int(chunks[pos[0]]) * S * 16 + slab * 16
+                    assert ci[blk] == k0 and block_row[blk] == br
+                    used[blk] += 1
+                    Cd[br * 16:br * 16 + 16] += blocks[blk] @ Bd[k0:k0 + 16]
+            assert cur == chunks.size - 1 and in_chunk >= 2
+    assert np.all(used == 1), "a block is multiplied zero or several times"
+    # read-ahead: the descriptors after the last op exist and are harmless
+    tail = plan["ops"][plan["n_ops"]:]
+    assert tail.shape[0] == PAD and np.all(tail[:, 0] == 0) and np.all(tail[:, 1] == (ZERO_HI | ZERO_LO)) and np.all(tail[:, 2] == 0)
+    return Cd
+
+
+def dense_of(A):
+    M, K, rp, ci = A["M"], A["K"], A["b_row_ptr"], A["b_col_idx"]
+    D = np.zeros((M, K))
+    blocks = A["b_val"].view(np.float16).astype(np.float64).reshape(-1, 16, 16)
+    rows = np.repeat(np.arange(M // 16), np.diff(rp))
+    for b, (r, c) in enumerate(zip(rows, ci)):
+        D[r * 16:r * 16 + 16, c:c + 16] = blocks[b]
+    return D
+
+
+def random_mask_matrix(mb, kb, density, seed, empty_rows=(), long_rows=()):
+    rng = np.random.default_rng(seed)
+    mask = rng.random((mb, kb)) < density
+    for r in empty_rows:
+        mask[r] = False
+    for r in long_rows:
+        mask[r] = True
+    if mask.sum() < 2:
+        mask[0, :2] = True
+    rp = np.concatenate([[0], np.cumsum(mask.sum(1))]).astype(np.int32)
+    ci = (np.nonzero(mask)[1] * 16).astype(np.int32)
+    val = gen.f16_bits(rng.normal(size=ci.size * 256))
+    return {"M": mb * 16, "K": kb * 16, "b_row_ptr": rp, "b_col_idx": ci, "b_val": val, "nnzb": ci.size}
+
+
+@pytest.mark.parametrize("mb,kb,density,seed", [(64, 64, 0.10, 1), (70, 40, 0.30, 2), (130, 100, 0.05, 3), (8, 200, 0.5, 4),
+                                                 (64, 16, 1.0, 5), (200, 33, 0.02, 6), (3, 3, 1.0, 7)])
+def test_replay_gives_a_times_b(mb, kb, density, seed):
+    A = random_mask_matrix(mb, kb, density, seed, empty_rows=(1,) if mb > 2 else (), long_rows=(2,) if mb > 3 else ())
+    plan = sweep_plan(A["b_row_ptr"], A["b_col_idx"], A["M"], A["K"])
+    rng = np.random.default_rng(seed + 100)
+    Bd = rng.normal(size=(A["K"], 8))
+    Cd = replay(plan, A, Bd)
+    assert np.allclose(Cd, dense_of(A) @ Bd, rtol=1e-12, atol=1e-12)
+    assert plan["pairs"] * 2 + plan["singles"] == A["nnzb"]
+    assert plan["n_ops"] == plan["pairs"] + plan["singles"] + plan["fillers"]
+
+
+def test_single_last_block_is_listed_as_second_half():
+    """An unpaired block at the very end of vals must not make the kernel read past the array."""
+    mask = np.zeros((2, 40), bool)
+    mask[0, [0, 1]] = True
+    mask[1, [39]] = True  # last block of the matrix, alone in its row
+    rp = np.concatenate([[0], np.cumsum(mask.sum(1))]).astype(np.int32)
+    ci = (np.nonzero(mask)[1] * 16).astype(np.int32)
+    A = {"M": 32, "K": 640, "b_row_ptr": rp, "b_col_idx": ci, "b_val": gen.f16_bits(np.ones(ci.size * 256)), "nnzb": ci.size}
+    plan = sweep_plan(rp, ci, 32, 640)
+    real = plan["ops"][:plan["n_ops"]]
+    lo = real[(real[:, 1] & ZERO_LO != 0) & (real[:, 1] & ZERO_HI == 0)]
+    assert lo.shape[0] == 1 and lo[0, 0] == (ci.size - 2) * 512
+    Cd = replay(plan, A, np.ones((640, 8)))
+    assert np.allclose(Cd, dense_of(A) @ np.ones((640, 8)))
+
+
+def test_headline_matrix_pairs_nearly_everything():
+    A = gen.block_pruned(8192, 0.10, 0.02)
+    plan = sweep_plan(A["b_row_ptr"], A["b_col_idx"], A["M"], A["K"])
+    assert plan["pairs"] * 2 + plan["singles"] == A["nnzb"]
+    # blocks paired inside a chunk or across two consecutive chunks: few stay single, hardly any filler
+    assert plan["singles"] < 0.12 * A["nnzb"] and plan["fillers"] < 0.001 * plan["n_ops"]
+    per_wave = np.diff(plan["op_ptr"])
+    assert per_wave.min() >= 2 * 32 and per_wave.max() <= 72 * 32
