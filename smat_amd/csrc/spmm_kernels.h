@@ -45,9 +45,9 @@ struct SpmmArgs {
 // the same K chunk or in two consecutive chunks of the row group's chunk list.
 //   w0 = byte offset of block q in vals (q * 512)
 //   w1 = LDS byte offset (inside the ring of stages) of the 16 rows of B under block q
-//        | flags in bits 0-2 | local block row 0..7 << 28
-//   w2 = the same offset for block q + 1
-//   w3 = 0
+//   w2 = offset of the rows under block q + 1, minus w1 (signed)
+//   w3 = flags in bits 0-2 | (local block row 0..7) * 40 << 23  (40 = bytes of code per block row in the
+//        kernel's computed jump to the MFMAs of that row)
 // LDS offset of ring slot s = (position of the chunk in the row group's chunk list % SWEEP_STAGES) *
 // SWEEP_S + block column inside the chunk:  (s / 8) * 16384 + (s % 8) * 32.
 // SWEEP_OP_ZERO_HI: block q + 1 does not belong to the op (unpaired block): its half is multiplied
@@ -61,7 +61,6 @@ struct SweepOp {
 constexpr uint32_t SWEEP_OP_ZERO_HI = 1u << 0;
 constexpr uint32_t SWEEP_OP_ZERO_LO = 1u << 1;
 constexpr uint32_t SWEEP_OP_BOUNDARY = 1u << 2;
-constexpr uint32_t SWEEP_LDS_MASK = 0x1C0E0u; // bits of an LDS offset in w1
 
 // Geometry of the sweep kernel (fixed at compile time).
 constexpr int SWEEP_TN = 4;     // n-tiles of 16 per workgroup panel -> 64 columns

@@ -59,8 +59,8 @@ constexpr int DA = 6;                                 // A operand ring (registe
 constexpr int AHEAD = 4;                              // A operands are loaded AHEAD ops ahead (< DA)
 constexpr int DQ = 6;                                 // op descriptors are read from LDS DQ ops ahead (ring of DQ scalar pairs)
 constexpr int UNROLL = 6;                             // multiple of PB + 1, DA and DQ
-constexpr int WIN_SLOTS = 3;                          // descriptor windows (64 ops, 1 KiB) resident per wavefront
-constexpr int WINDOW_BYTES = W * WIN_SLOTS * 1024;    // 24 KiB
+constexpr int WIN_SLOTS = 4;                          // descriptor windows (64 ops, 1 KiB) per wavefront in LDS; three are in use
+constexpr int WINDOW_BYTES = W * WIN_SLOTS * 1024;    // 32 KiB: with the four stages all 160 KiB of LDS
 static_assert(TN == 4 && RW == 8 && W == 8 && S == 16 && NS == 4 && COPIES == 4, "geometry the code below assumes");
 static_assert(UNROLL % (PB + 1) == 0 && UNROLL % DA == 0 && UNROLL % DQ == 0 && AHEAD < DA && AHEAD < DQ && PB < DQ,
               "register sets are addressed by the unroll position");
@@ -89,20 +89,6 @@ __device__ __forceinline__ void zero_accumulators()
                    "a115", "a116", "a117", "a118", "a119", "a120", "a121", "a122", "a123", "a124", "a125", "a126", "a127");
 #undef Z16
 #undef Z4
-}
-
-// The four MFMAs of one op on block row R of the wavefront: a[16R + 4t .. + 3] += b[t] x a.
-template <int R>
-__device__ __forceinline__ void mfma_row(const f16x8 (&b)[TN], const f16x8 &a)
-{
-    asm volatile("s_nop 1\n\t"
-                 "v_mfma_f32_16x16x32_f16 a[%5:%6], %0, %4, a[%5:%6]\n\t"
-                 "v_mfma_f32_16x16x32_f16 a[%7:%8], %1, %4, a[%7:%8]\n\t"
-                 "v_mfma_f32_16x16x32_f16 a[%9:%10], %2, %4, a[%9:%10]\n\t"
-                 "v_mfma_f32_16x16x32_f16 a[%11:%12], %3, %4, a[%11:%12]"
-                 :
-                 : "v"(b[0]), "v"(b[1]), "v"(b[2]), "v"(b[3]), "v"(a), "n"(16 * R), "n"(16 * R + 3), "n"(16 * R + 4), "n"(16 * R + 7),
-                   "n"(16 * R + 8), "n"(16 * R + 11), "n"(16 * R + 12), "n"(16 * R + 15));
 }
 
 // Reads accumulator tile (R, T) after the last MFMA has retired.
@@ -152,7 +138,6 @@ __global__ __launch_bounds__(THREADS) void spmm_sweep_kernel(
     const uint32_t lbase = (uint32_t)(uintptr_t)(__attribute__((address_space(3))) void *)lds;
     // column (within the panel) of MFMA row i16 in n-tile 0 is 16*(i16>>2) + (i16&3); n-tile t adds 4*t.
     // The swizzle value of every such column equals i16.
-    const uint32_t rd_lane = (uint32_t)(16 * (i16 >> 2) + (i16 & 3)) * ROW_BYTES; // byte offset in a stage
     const uint32_t lane_xor = (uint32_t)((kh ^ i16) << 4); // ((2*slab | kh) ^ i16) << 4 == (slab * 32) ^ lane_xor
     const uint32_t a_lane_bytes = (uint32_t)(i16 * 16 + kh * 8) * 2u; // this lane's 16 bytes inside a block
 
@@ -173,188 +158,57 @@ __global__ __launch_bounds__(THREADS) void spmm_sweep_kernel(
     const int n_ops = op_ptr[rg * W + wave + 1] - op_begin;
 
     if (n_chunks > 0) { // uniform over the workgroup: every wavefront has the chunk list of its row group
-        // Vector memory instructions complete in order.  `age` counts the ops (= A loads) since the last chunk
-        // boundary, `burst` the copy instructions issued at that boundary: together they give the immediate of
-        // every vmcnt wait.
-        int age = 0, burst = 0;
         auto lds_copy = [&](uint32_t voff, const void *sbase, uint32_t dst) { // 64 lanes x 16 B -> LDS dst + lane * 16
             asm volatile("s_mov_b32 m0, %2\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, %1"
                          :
                          : "v"(voff), "s"(sbase), "s"(dst)
                          : "memory");
-            burst++;
         };
-
         // ---- B panel copies: this wavefront fills rows ((wave & 3) * 4 + it) * 4 .. + 3 of slab group wave / 4 ----
         // lane -> (row q = lane / 16, physical slot ps = lane % 16); logical slot = ps ^ swizzle(n),
         // swizzle(n) = (n & 3) | ((n >> 2) & 12) = q | (wave & 3) << 2 for these rows.
         const int q = lane >> 4;
         const uint32_t ls = (uint32_t)((lane & 15) ^ (q | ((wave & 3) << 2)));
-        const uint32_t k_lane = (uint32_t)(wave >> 2) * 128u + ls * 8u; // k inside the chunk
-        const uint32_t col_lane = (uint32_t)q * (uint32_t)K;            // elements; the launcher checks K < 2^28
+        const uint32_t k_lane = (uint32_t)(wave >> 2) * 128u + ls * 8u;  // k inside the chunk
+        const uint32_t col_bytes = (uint32_t)q * (uint32_t)K * 2u;       // the launcher checks K < 2^28
         const uint32_t kmax = (uint32_t)K - 8u;
-        auto issue_copies = [&](int cl) {
-            const uint32_t k0 = (uint32_t)chunk_ids[c_begin + cl] * (uint32_t)(S * 16);
-            uint32_t k = k0 + k_lane;
+        const uint32_t dst_wave = lbase + (uint32_t)(wave * COPIES) * 1024u;
+        // the four copy instructions of a chunk: scalar base = first of their four columns of B, bit `it` of
+        // copy_mask = those columns exist (N % 8 == 0: all four or none)
+        const int col0 = n0 + (wave & 3) * 16;
+        const uint16_t *sb0 = B + (long)(col0 + 0) * K, *sb1 = B + (long)(col0 + 4) * K;
+        const uint16_t *sb2 = B + (long)(col0 + 8) * K, *sb3 = B + (long)(col0 + 12) * K;
+        const uint32_t copy_mask = __builtin_amdgcn_readfirstlane(
+            (col0 < N ? 1u : 0u) | (col0 + 4 < N ? 2u : 0u) | (col0 + 8 < N ? 4u : 0u) | (col0 + 12 < N ? 8u : 0u));
+        const int32_t *chunk_ptr = chunk_ids + c_begin;
+        auto issue_copies = [&](int cl) { // chunk cl of the row group's list into stage cl % NS
+            uint32_t k = (uint32_t)chunk_ptr[cl] * (uint32_t)(S * 16) + k_lane;
             k = k < kmax ? k : kmax; // slabs past K are referenced by no op; keep the read inside the matrix
-            const uint32_t voff = (col_lane + k) * 2u;
-            const uint32_t dst0 = lbase + (uint32_t)(cl % NS) * STAGE_BYTES + (uint32_t)(wave * COPIES) * 1024u;
-#pragma unroll
-            for (int it = 0; it < COPIES; it++) {
-                const int row4 = ((wave & 3) * 4 + it) * 4; // first of four columns, wave-uniform
-                if (n0 + row4 >= N) continue;               // N % 8 == 0: all four columns or none
-                lds_copy(voff, B + (long)(n0 + row4) * K, dst0 + (uint32_t)it * 1024u);
-            }
+            const uint32_t voff = col_bytes + k * 2u;
+            const uint32_t dst0 = dst_wave + (uint32_t)(cl % NS) * STAGE_BYTES;
+            if (copy_mask & 1) lds_copy(voff, sb0, dst0);
+            if (copy_mask & 2) lds_copy(voff, sb1, dst0 + 1024u);
+            if (copy_mask & 4) lds_copy(voff, sb2, dst0 + 2048u);
+            if (copy_mask & 8) lds_copy(voff, sb3, dst0 + 3072u);
         };
-
-        // ---- op descriptors: windows of 64 ops (1 KiB, one copy instruction) in three LDS slots per wavefront ----
+        // ---- op descriptors: windows of 64 ops (1 KiB, one copy instruction), four LDS slots per wavefront ----
         const SweepOp *op_base = ops + op_begin; // the plan pads the array: reads past n_ops stay inside it
-        const uint32_t win_base = (uint32_t)(NS * STAGE_BYTES) + (uint32_t)wave * (WIN_SLOTS * 1024u); // byte offset in LDS
-        int win_next = 0; // first window not requested yet
-        auto copy_window = [&]() {
-            lds_copy((uint32_t)lane * 16u, op_base + (long)win_next * 64, lbase + win_base + (uint32_t)(win_next % WIN_SLOTS) * 1024u);
-            win_next++;
-        };
-        // plain LDS read, same address in every lane; made scalar where it is used, several ops later
-        auto read_desc = [&](int x) {
-            return *reinterpret_cast<const uint4 *>(lds + win_base + (uint32_t)((x >> 6) % WIN_SLOTS) * 1024u + (uint32_t)(x & 63) * 16u);
-        };
-
-        // ---- operand registers ----
-        f16x8 bq[PB + 1][TN];
-        f16x8 aq[DA];
-        uint4 dq[DQ];      // descriptors of ops i .. i + DQ - 1 (slot = op % DQ), one copy per lane
-        uint32_t fq[PB + 1]; // flags and block row (word 1) of the ops whose B operands are under way
-        const f16x8 zero8 = {0, 0, 0, 0, 0, 0, 0, 0};
-        // A operand: one buffer load of the 1 KiB pair, lanes 32-63 take the second block.  Where a block does not
-        // belong to the op its lanes get an offset past the end of the buffer, for which the load returns zeros:
-        // between the load and the MFMAs nothing touches the operand registers.
-        const uint32_t a_voff = (uint32_t)sel * 512u + a_lane_bytes;
-        const uint32_t a_voff_zero_hi = sel ? 0x80000000u : a_voff;
-        const uint32_t a_voff_zero_lo = sel ? a_voff : 0x80000000u;
-        const uint32_t a_voff_zero = 0x80000000u;
-
-        // reads the B operands of an op: lanes 0-31 from the slab of its first block, 32-63 of the second
-        auto issue_b = [&](f16x8(&b)[TN], uint32_t w1, uint32_t w2) {
-            const uint32_t off0 = w1 & SWEEP_LDS_MASK, off1 = w2;
-            const unsigned char *p = lds + rd_lane + ((sel ? off1 : off0) ^ lane_xor);
-#pragma unroll
-            for (int tt = 0; tt < TN; tt++) b[tt] = *reinterpret_cast<const f16x8 *>(p + tt * 4 * ROW_BYTES);
-        };
-        // loads the A operand of an op: its two blocks are neighbours in vals, 1 KiB in MFMA operand order
-        auto issue_a = [&](f16x8 &a, uint32_t w0, uint32_t w1) {
-            const uint32_t z = w1 & (SWEEP_OP_ZERO_HI | SWEEP_OP_ZERO_LO);
-            if (z == 0)
-                asm volatile("buffer_load_dwordx4 %0, %1, %2, %3 offen" : "=v"(a) : "v"(a_voff), "s"(vals_rsrc), "s"(w0));
-            else if (z == SWEEP_OP_ZERO_HI)
-                asm volatile("buffer_load_dwordx4 %0, %1, %2, %3 offen" : "=v"(a) : "v"(a_voff_zero_hi), "s"(vals_rsrc), "s"(w0));
-            else if (z == SWEEP_OP_ZERO_LO)
-                asm volatile("buffer_load_dwordx4 %0, %1, %2, %3 offen" : "=v"(a) : "v"(a_voff_zero_lo), "s"(vals_rsrc), "s"(w0));
-            else
-                asm volatile("buffer_load_dwordx4 %0, %1, %2, %3 offen" : "=v"(a) : "v"(a_voff_zero), "s"(vals_rsrc), "s"(w0));
-        };
-
-        // ---- prologue: chunks 0 and 1 resident, descriptors of the first 192 ops, first operands under way ----
+        const uint32_t win_lds = lbase + (uint32_t)(NS * STAGE_BYTES) + (uint32_t)wave * (WIN_SLOTS * 1024u);
+        const uint32_t lane16 = (uint32_t)lane * 16u;
+        // ---- prologue: chunks 0 and 1 and the descriptors of the first 192 ops resident ----
         issue_copies(0);
         if (n_chunks > 1) issue_copies(1);
-        copy_window();
-        copy_window();
-        copy_window();
+        for (int wdw = 0; wdw < 3; wdw++) lds_copy(lane16, op_base + (long)wdw * 64, win_lds + (uint32_t)wdw * 1024u);
         asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
         __syncthreads();
-#pragma unroll
-        for (int d = 0; d < DQ; d++) dq[d] = read_desc(d);
-#pragma unroll
-        for (int d = 0; d < AHEAD; d++)
-            issue_a(aq[d], __builtin_amdgcn_readfirstlane(dq[d].x), __builtin_amdgcn_readfirstlane(dq[d].y));
-        burst = 0;
-        if (n_chunks > 2) issue_copies(2); // after the first A loads, like the copies of a boundary
-#pragma unroll
-        for (int d = AHEAD; d < DA; d++) aq[d] = zero8;
-#pragma unroll
-        for (int d = 0; d < PB; d++) {
-            fq[d] = __builtin_amdgcn_readfirstlane(dq[d].y);
-            issue_b(bq[d], fq[d], __builtin_amdgcn_readfirstlane(dq[d].z));
-        }
-        fq[PB] = 0;
-#pragma unroll
-        for (int tt = 0; tt < TN; tt++) bq[PB][tt] = zero8;
 
-        int cur = 0; // chunk (index into the row group's chunk list) the executed ops belong to
-        int i = 0;   // op executed next
-
-        // One op.  J = i % UNROLL selects the register sets.
-        auto step = [&](auto jc) {
-            constexpr int J = decltype(jc)::value;
-            const uint32_t w1 = fq[J % (PB + 1)];
-            if (w1 & SWEEP_OP_BOUNDARY) {
-                // entering chunk cur: the copies of chunk cur + 1 (issued when chunk cur - 1 was entered, `age` A
-                // loads ago) have landed; after the barrier every wavefront is done with chunk cur - 1, and the
-                // stage of chunk cur - 2 takes the copies of chunk cur + 2
-                cur++;
-                if (age <= AHEAD) { // else an A load issued after them has been waited for
-                    if (age == 2) asm volatile("s_waitcnt vmcnt(2)" ::: "memory");
-                    else if (age == 3) asm volatile("s_waitcnt vmcnt(3)" ::: "memory");
-                    else if (age == 4) asm volatile("s_waitcnt vmcnt(4)" ::: "memory");
-                    else asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
-                }
-                asm volatile("s_barrier" ::: "memory");
-                burst = 0;
-                age = 0;
-                if (cur + 2 < n_chunks) issue_copies(cur + 2);
-                // descriptor windows: those up to two ahead of the current op are requested here; a chunk holds
-                // at most 72 ops of a wavefront, so a window is requested at least 50 ops before its first read
-                // and the windows requested at the last boundary cover the read-ahead past the last op
-                while ((i >> 6) + 2 >= win_next) copy_window();
-            }
-            // Operands of later ops.  Unconditional: past the end of the stream the descriptors are the plan's
-            // padding (block 0, first slab), whose operands are fetched and never used.  A condition here would
-            // make the compiler wait for every LDS read before the MFMAs (it has to assume the path on which
-            // the younger reads were not issued).
-            {
-                const uint4 &db = dq[(J + PB) % DQ];
-                fq[(J + PB) % (PB + 1)] = __builtin_amdgcn_readfirstlane(db.y);
-                issue_b(bq[(J + PB) % (PB + 1)], fq[(J + PB) % (PB + 1)], __builtin_amdgcn_readfirstlane(db.z));
-                const uint4 &da = dq[(J + AHEAD) % DQ];
-                issue_a(aq[(J + AHEAD) % DA], __builtin_amdgcn_readfirstlane(da.x), __builtin_amdgcn_readfirstlane(da.y));
-                dq[J % DQ] = read_desc(i + DQ); // replaces the descriptor of op i, whose word 1 is in w1
-            }
-            __builtin_amdgcn_sched_barrier(0);
-            // the A operand of op i: AHEAD younger A loads, and the copies of the last boundary if that young
-            // (the waits carry no operands: an operand tied to the wait lets the compiler copy the register
-            // before it; the operand registers go from the load straight to the MFMAs)
-            if (age < AHEAD) {
-                if (burst == COPIES) asm volatile("s_waitcnt vmcnt(8)" ::: "memory");
-                else if (burst == COPIES + 1) asm volatile("s_waitcnt vmcnt(9)" ::: "memory");
-                else if (burst == COPIES + 2) asm volatile("s_waitcnt vmcnt(10)" ::: "memory");
-                else asm volatile("s_waitcnt vmcnt(4)" ::: "memory"); // fewer copies (last panel, last chunks): waits for them too
-            } else {
-                asm volatile("s_waitcnt vmcnt(4)" ::: "memory");
-            }
-            static_assert(AHEAD == 4 && COPIES == 4, "immediates above");
-            age++;
-            const f16x8 &av = aq[J % DA];
-            f16x8(&bc)[TN] = bq[J % (PB + 1)];
-            switch (w1 >> 28) {
-            case 0: mfma_row<0>(bc, av); break;
-            case 1: mfma_row<1>(bc, av); break;
-            case 2: mfma_row<2>(bc, av); break;
-            case 3: mfma_row<3>(bc, av); break;
-            case 4: mfma_row<4>(bc, av); break;
-            case 5: mfma_row<5>(bc, av); break;
-            case 6: mfma_row<6>(bc, av); break;
-            default: mfma_row<7>(bc, av); break;
-            }
-        };
-        while (i < n_ops) {
-            step(std::integral_constant<int, 0>{}); if (++i >= n_ops) break;
-            step(std::integral_constant<int, 1>{}); if (++i >= n_ops) break;
-            step(std::integral_constant<int, 2>{}); if (++i >= n_ops) break;
-            step(std::integral_constant<int, 3>{}); if (++i >= n_ops) break;
-            step(std::integral_constant<int, 4>{}); if (++i >= n_ops) break;
-            step(std::integral_constant<int, 5>{}); ++i;
-        }
-        asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+        // ---- the main loop: see gen_sweep_loop.py ----
+        const uint32_t rd_addr = lbase + (uint32_t)(16 * (i16 >> 2) + (i16 & 3)) * ROW_BYTES; // LDS address of this lane's column in stage 0
+        const uint32_t a_voff = (uint32_t)sel * 512u + a_lane_bytes; // lanes 32-63 take the second block of the pair
+        const uint32_t sel01 = (uint32_t)sel;
+        const uint32_t n_ops_u = __builtin_amdgcn_readfirstlane((uint32_t)n_ops), n_chunks_u = __builtin_amdgcn_readfirstlane((uint32_t)n_chunks);
+        const uint32_t op_lo = (uint32_t)(uintptr_t)op_base, op_hi = (uint32_t)((uintptr_t)op_base >> 32);
+#include "spmm_sweep_loop.inc"
     }
     asm volatile("s_nop 15\n\ts_nop 15" ::: "memory"); // the last MFMAs retire before their results are read
 

@@ -13,6 +13,7 @@ namespace {
 // mirrors spmm_kernels.h (that header needs the HIP runtime; this file is compiled by g++)
 constexpr uint32_t OP_ZERO_HI = 1u << 0, OP_ZERO_LO = 1u << 1, OP_BOUNDARY = 1u << 2;
 constexpr int G = 64, RW = 8, WAVES = 8, S = 16, STAGES = 4, MIN_OPS = 2, OP_PAD = 384;
+constexpr uint32_t ROW_CODE = 40; // bytes of code per block row in the kernel's MFMA dispatch
 
 // LDS byte offset of the 16 rows of B under a block: chunk position in the row group's list, block column in the chunk
 uint32_t lds_offset(int32_t chunk_pos, int32_t slab)
@@ -65,8 +66,9 @@ void build_sweep_plan(const int32_t *row_ptr, const int32_t *col_idx, size_t mb,
                         const int32_t cl1 = local[(size_t)bc1 / S];
                         if (cl1 - cl0 <= 1) { // same chunk or the next listed one: both stages are resident
                             op.w0 = (uint32_t)q * 512u;
-                            op.w1 = off0 | ((uint32_t)r << 28);
-                            op.w2 = lds_offset(cl1, bc1 % S);
+                            op.w1 = off0;
+                            op.w2 = lds_offset(cl1, bc1 % S) - off0;
+                            op.w3 = (uint32_t)r * ROW_CODE << 23;
                             exec = cl1;
                             pair = true;
                         }
@@ -74,13 +76,13 @@ void build_sweep_plan(const int32_t *row_ptr, const int32_t *col_idx, size_t mb,
                     if (!pair) {
                         if (q + 1 < nnzb) { // blocks (q, q + 1), the second multiplied by zeros
                             op.w0 = (uint32_t)q * 512u;
-                            op.w1 = off0 | OP_ZERO_HI | ((uint32_t)r << 28);
-                            op.w2 = off0;
+                            op.w3 = OP_ZERO_HI | ((uint32_t)r * ROW_CODE << 23);
                         } else { // last block of the matrix: blocks (q - 1, q), the first multiplied by zeros
                             op.w0 = (uint32_t)(q - 1) * 512u;
-                            op.w1 = off0 | OP_ZERO_LO | ((uint32_t)r << 28);
-                            op.w2 = off0;
+                            op.w3 = OP_ZERO_LO | ((uint32_t)r * ROW_CODE << 23);
                         }
+                        op.w1 = off0; // both halves read the rows of B under this block
+                        op.w2 = 0;
                     }
                     (pair ? out.n_pairs : out.n_singles)++;
                     // rank = how many ops of this block row the chunk already holds: ops of one block
@@ -99,10 +101,10 @@ void build_sweep_plan(const int32_t *row_ptr, const int32_t *col_idx, size_t mb,
                 });
                 while (list.size() < (size_t)MIN_OPS) { // filler: blocks 0 and 1 times zeros, first slab of this chunk
                     const uint32_t off = lds_offset((int32_t)c, 0);
-                    list.push_back(Ranked{0, 0, SweepOpHost{0, off | OP_ZERO_HI | OP_ZERO_LO, off, 0}});
+                    list.push_back(Ranked{0, 0, SweepOpHost{0, off, 0, OP_ZERO_HI | OP_ZERO_LO}});
                     out.n_fillers++;
                 }
-                if (c > 0) list[0].op.w1 |= OP_BOUNDARY;
+                if (c > 0) list[0].op.w3 |= OP_BOUNDARY;
                 for (const Ranked &x : list) out.ops.push_back(x.op);
             }
         }
@@ -110,7 +112,7 @@ void build_sweep_plan(const int32_t *row_ptr, const int32_t *col_idx, size_t mb,
     }
     out.op_ptr.push_back((int32_t)out.ops.size());
     // what the kernel reads ahead of the last op: fetched, never executed
-    out.ops.resize(out.ops.size() + OP_PAD, SweepOpHost{0, OP_ZERO_HI | OP_ZERO_LO, 0, 0});
+    out.ops.resize(out.ops.size() + OP_PAD, SweepOpHost{0, 0, 0, OP_ZERO_HI | OP_ZERO_LO});
 }
 
 } // namespace smat

@@ -67,15 +67,18 @@ def replay(plan, A, Bd):
                 continue
             cur, in_chunk = 0, 0
             for w0, w1, w2, w3 in ops:
-                if w1 & BOUNDARY:
+                if w3 & BOUNDARY:
                     assert in_chunk >= 2, "fewer than two ops in a chunk"
                     cur, in_chunk = cur + 1, 0
                 in_chunk += 1
                 q = int(w0) // 512
-                assert int(w0) % 512 == 0 and 0 <= q and q + 1 < nnzb and w3 == 0
-                r = int(w1) >> 28
+                assert int(w0) % 512 == 0 and 0 <= q and q + 1 < nnzb and int(w3) & 0x7FFFF8 == 0
+                assert (int(w3) >> 23) % 40 == 0
+                r = (int(w3) >> 23) // 40
+                assert r < RW
                 br = rg * G + w * RW + r
-                for half, (off, zero) in enumerate(((int(w1) & LDS_MASK, w1 & ZERO_LO), (int(w2), w1 & ZERO_HI))):
+                off1 = (int(w1) + int(np.int32(w2))) & 0xFFFFFFFF
+                for half, (off, zero) in enumerate(((int(w1), w3 & ZERO_LO), (off1, w3 & ZERO_HI))):
                     stage, slab = slot_of(off)
                     # the stage holds chunk position cur or cur - 1 (whichever maps to it); cur + 1 is also
                     # resident but no op may use it yet
@@ -92,7 +95,7 @@ def replay(plan, A, Bd):
     assert np.all(used == 1), "a block is multiplied zero or several times"
     # read-ahead: the descriptors after the last op exist and are harmless
     tail = plan["ops"][plan["n_ops"]:]
-    assert tail.shape[0] == PAD and np.all(tail[:, 0] == 0) and np.all(tail[:, 1] == (ZERO_HI | ZERO_LO)) and np.all(tail[:, 2] == 0)
+    assert tail.shape[0] == PAD and np.all(tail[:, :3] == 0) and np.all(tail[:, 3] == (ZERO_HI | ZERO_LO))
     return Cd
 
 
@@ -144,7 +147,7 @@ def test_single_last_block_is_listed_as_second_half():
     A = {"M": 32, "K": 640, "b_row_ptr": rp, "b_col_idx": ci, "b_val": gen.f16_bits(np.ones(ci.size * 256)), "nnzb": ci.size}
     plan = sweep_plan(rp, ci, 32, 640)
     real = plan["ops"][:plan["n_ops"]]
-    lo = real[(real[:, 1] & ZERO_LO != 0) & (real[:, 1] & ZERO_HI == 0)]
+    lo = real[(real[:, 3] & ZERO_LO != 0) & (real[:, 3] & ZERO_HI == 0)]
     assert lo.shape[0] == 1 and lo[0, 0] == (ci.size - 2) * 512
     Cd = replay(plan, A, np.ones((640, 8)))
     assert np.allclose(Cd, dense_of(A) @ np.ones((640, 8)))
