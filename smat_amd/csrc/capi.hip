@@ -39,7 +39,7 @@ struct smat_plan {
     uint16_t *d_bpack = nullptr; // slab-major copy of B, K * n_cap halves (row-wise kernel, when it pays)
     // sweep kernel work list (present when kernel == SMAT_KERNEL_SWEEP)
     int n_rg = 0, n_records = 0, n_ops = 0;
-    int32_t *d_rg_chunk_ptr = nullptr, *d_chunk_ids = nullptr, *d_op_ptr = nullptr;
+    int32_t *d_rg_chunk_ptr = nullptr, *d_chunk_ids = nullptr, *d_op_ptr = nullptr, *d_row_map = nullptr;
     SweepOp *d_ops = nullptr;
     // compacted-column kernel (present after smat_plan_attach_values)
     CompactPlan *compact = nullptr;
@@ -142,7 +142,7 @@ extern "C" int smat_spmm_bcsr_f16_ex(const uint16_t *vals, const int32_t *row_pt
         SweepArgs w{};
         w.vals = vals; w.B = B; w.C = C; w.M = M; w.N = N; w.K = K; w.nnzb = nnzb; w.c_f32 = a.c_f32;
         w.rg_chunk_ptr = plan->d_rg_chunk_ptr; w.chunk_ids = plan->d_chunk_ids;
-        w.op_ptr = plan->d_op_ptr; w.ops = plan->d_ops; w.n_rg = plan->n_rg;
+        w.op_ptr = plan->d_op_ptr; w.ops = plan->d_ops; w.row_map = plan->d_row_map; w.n_rg = plan->n_rg;
         e = launch_sweep(w, static_cast<hipStream_t>(o.stream));
     } else {
         e = launch_rowwise(a, static_cast<hipStream_t>(o.stream));
@@ -280,6 +280,7 @@ extern "C" int smat_plan_create(smat_plan **out, const int32_t *row_ptr_host,
         upload((void **)&p->d_rg_chunk_ptr, h.rg_chunk_ptr.data(), h.rg_chunk_ptr.size() * sizeof(int32_t));
         upload((void **)&p->d_chunk_ids, h.chunk_ids.data(), h.chunk_ids.size() * sizeof(int32_t));
         upload((void **)&p->d_op_ptr, h.op_ptr.data(), h.op_ptr.size() * sizeof(int32_t));
+        upload((void **)&p->d_row_map, h.row_map.data(), h.row_map.size() * sizeof(int32_t));
         static_assert(sizeof(SweepOpHost) == sizeof(SweepOp), "host and device op layouts");
         upload((void **)&p->d_ops, h.ops.data(), h.ops.size() * sizeof(SweepOp));
         if (p->d_bpack && want != SMAT_KERNEL_ROWWISE_PACKED) { // the sweep kernel reads B in place
@@ -341,6 +342,7 @@ extern "C" int smat_plan_destroy(smat_plan *p)
     if (p->d_rg_chunk_ptr) (void)hipFree(p->d_rg_chunk_ptr);
     if (p->d_chunk_ids) (void)hipFree(p->d_chunk_ids);
     if (p->d_op_ptr) (void)hipFree(p->d_op_ptr);
+    if (p->d_row_map) (void)hipFree(p->d_row_map);
     if (p->d_ops) (void)hipFree(p->d_ops);
     delete p;
     return SMAT_OK;

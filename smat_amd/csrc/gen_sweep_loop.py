@@ -10,22 +10,38 @@ the six positions of the register rings and numbers the registers; run it after 
     python3 gen_sweep_loop.py > spmm_sweep_loop.inc
 
 Registers (fixed, all listed as clobbers):
+    (with the default ring of six)
     v40-v87    B operands, three sets of 4 tiles x 4 registers (op i uses set i % 3)
     v88-v111   A operands, ring of six (op i uses slot i % 6)
-    v112-v115  descriptor being read from LDS
-    v120-v127  temporaries; v124-v126 = A offsets with the upper / lower / both halves out of range
+    v112-v119  two descriptors being read from LDS
+    v120-v126  temporaries; v124-v126 = A offsets with the upper / lower / both halves out of range
     s40..      loop state, s52-s75 descriptor ring (op i in slot i % 6: w0 w1 w2 w3)
     a0-a127    accumulators (block row r, tile t in a[16r + 4t .. + 3])
 """
 
-UNROLL = 6
-AHEAD = 4      # A operands are loaded AHEAD ops ahead
+import argparse
+
+ap = argparse.ArgumentParser()
+ap.add_argument("--unroll", type=int, default=6, help="ring positions: A ring slots = descriptor ring slots; multiple of 6")
+ap.add_argument("--ahead", type=int, default=4, help="A operands are loaded this many ops ahead (< unroll)")
+ap.add_argument("--ablate", default="", help="timing experiments only, wrong results: any of a,copy,barrier,mfma,bread")
+args = ap.parse_args()
+UNROLL = args.unroll
+AHEAD = args.ahead
 PB = 2         # B operands are read PB ops ahead
-DQ = 6         # descriptors are read DQ ops ahead (and made scalar one op later)
+DQ = UNROLL    # descriptor ring slots; a descriptor is read DQ + 1 ops ahead and made scalar two ops later
+ABL = set(x for x in args.ablate.split(",") if x)
+assert UNROLL % (PB + 1) == 0 and UNROLL % 2 == 0 and PB < AHEAD < UNROLL
 
 S_I, S_AGE, S_BURST, S_CUR, S_WINNEXT, S_DP, S_T0, S_T1, S_T2, S_T3, S_T4, S_T5 = range(40, 52)
 RING0 = 52     # s[52 + 4*slot + word]
-V_B0, V_A0, V_DESC, V_T0, V_T1, V_T2, V_COPY, V_AZH, V_AZL, V_AZB = 40, 88, 112, 120, 121, 122, 123, 124, 125, 126
+assert RING0 + 4 * UNROLL <= 100
+V_TOP = 128
+V_T0, V_T1, V_T2, V_COPY, V_AZH, V_AZL, V_AZB = range(V_TOP - 8, V_TOP - 1)
+V_DESC = V_TOP - 16  # two buffers of four registers
+V_A0 = V_DESC - 4 * UNROLL
+V_B0 = V_A0 - 16 * (PB + 1)
+V_FIRST = V_B0
 
 
 def ring(slot, word):
@@ -55,6 +71,8 @@ def label(name):
 
 def a_load(dst_slot, desc_slot, tag):
     """A operand of the op whose descriptor sits in ring slot desc_slot."""
+    if "a" in ABL:
+        return
     emit(f"s_and_b32 s{S_T0}, {ring(desc_slot, 3)}, 3")          # which halves are zeros: SCC = any
     emit(f"s_cbranch_scc1 Lazero_{tag}_%=")
     emit(f"buffer_load_dwordx4 {aslot(dst_slot)}, %[a_voff], %[rsrc], {ring(desc_slot, 0)} offen")
@@ -62,6 +80,8 @@ def a_load(dst_slot, desc_slot, tag):
 
 
 def a_load_slow(dst_slot, desc_slot, tag):
+    if "a" in ABL:
+        return
     label(f"Lazero_{tag}")
     emit(f"s_cmp_eq_u32 s{S_T0}, 1")
     emit(f"s_cbranch_scc1 Lazh_{tag}_%=")
@@ -84,20 +104,25 @@ def b_reads(dst_set, desc_slot):
     emit(f"v_xad_u32 v{V_T2}, v{V_T1}, %[lane_xor], %[rd_lane]")
     for t in range(4):
         off = f" offset:{1024 * t}" if t else ""
+        if "bread" in ABL:
+            emit("s_nop 0")
+            continue
         emit(f"ds_read_b128 {bset(dst_set, t)}, v{V_T2}{off}")
 
 
-def desc_read():
+def desc_read(buf):
+    b = V_DESC + 4 * (buf % 2)
     emit(f"s_add_u32 s{S_DP}, s{S_DP}, 16")
     emit(f"s_and_b32 s{S_DP}, s{S_DP}, 0xfff")
     emit(f"s_add_u32 s{S_T0}, s{S_DP}, %[win_lds]")
     emit(f"v_mov_b32 v{V_T0}, s{S_T0}")
-    emit(f"ds_read_b128 v[{V_DESC}:{V_DESC + 3}], v{V_T0}")
+    emit(f"ds_read_b128 v[{b}:{b + 3}], v{V_T0}")
 
 
-def desc_scalar(slot):
+def desc_scalar(slot, buf):
+    b = V_DESC + 4 * (buf % 2)
     for w in range(4):
-        emit(f"v_readfirstlane_b32 {ring(slot, w)}, v{V_DESC + w}")
+        emit(f"v_readfirstlane_b32 {ring(slot, w)}, v{b + w}")
 
 
 def mfma_dispatch(J):
@@ -114,6 +139,10 @@ def mfma_dispatch(J):
         emit("s_nop 1")
         for t in range(4):
             acc = f"a[{16 * r + 4 * t}:{16 * r + 4 * t + 3}]"
+            if "mfma" in ABL:
+                emit("v_nop")
+                emit("v_nop")
+                continue
             emit(f"v_mfma_f32_16x16x32_f16 {acc}, {bset(J, t)}, {aslot(J)}, {acc}")
         if r < 7:
             emit(f"s_branch Lmdone_{J}_%=")
@@ -127,18 +156,20 @@ def boundary(J):
     # the copies were issued `age` A loads ago; beyond AHEAD one of those loads has been waited for already
     emit(f"s_cmp_gt_u32 s{S_AGE}, {AHEAD}")
     emit(f"s_cbranch_scc1 Lbw_{J}_%=")
-    for a in (2, 3, 4):
+    ages = list(range(2, AHEAD + 1))
+    for a in ages:
         emit(f"s_cmp_eq_u32 s{S_AGE}, {a}")
         emit(f"s_cbranch_scc1 Lbw{a}_{J}_%=")
     emit("s_waitcnt vmcnt(0)")
     emit(f"s_branch Lbw_{J}_%=")
-    for a in (2, 3, 4):
+    for a in ages:
         label(f"Lbw{a}_{J}")
         emit(f"s_waitcnt vmcnt({a})")
-        if a != 4:
+        if a != ages[-1]:
             emit(f"s_branch Lbw_{J}_%=")
     label(f"Lbw_{J}")
-    emit("s_barrier")
+    if "barrier" not in ABL:
+        emit("s_barrier")
     emit(f"s_mov_b32 s{S_BURST}, 0")
     emit(f"s_mov_b32 s{S_AGE}, 0")
     # copies of chunk cur + 2 into stage (cur + 2) % 4
@@ -160,8 +191,9 @@ def boundary(J):
         emit(f"s_cbranch_scc0 Lskip{it}_{J}_%=")
         emit(f"s_mov_b32 m0, s{S_T1}")
         emit("s_nop 0")
-        emit(f"global_load_lds_dwordx4 v{V_COPY}, %[sb{it}]")
-        emit(f"s_add_u32 s{S_BURST}, s{S_BURST}, 1")
+        if "copy" not in ABL:
+            emit(f"global_load_lds_dwordx4 v{V_COPY}, %[sb{it}]")
+            emit(f"s_add_u32 s{S_BURST}, s{S_BURST}, 1")
         label(f"Lskip{it}_{J}")
         if it < 3:
             emit(f"s_add_u32 s{S_T1}, s{S_T1}, 1024")
@@ -207,11 +239,12 @@ def step(J):
     emit(f"s_bitcmp1_b32 {ring(J, 3)}, 2")                       # first op of a chunk?
     emit(f"s_cbranch_scc1 Lbound_{J}_%=")
     label(f"Lbdone_{J}")
-    # LDS returns in order: per step one descriptor read, then four B reads.  Everything up to the
-    # descriptor read of the previous step is needed now (B operands of this op, descriptor of op i + 5).
-    emit("s_waitcnt lgkmcnt(4)")
-    desc_scalar(J + DQ - 1)
-    desc_read()
+    # LDS returns in order: per step one descriptor read, then four B reads.  What the step before the
+    # previous one issued is needed now (B operands of this op, descriptor of op i + DQ - 1); the five reads
+    # of the previous step may still be under way.
+    emit("s_waitcnt lgkmcnt(5)")
+    desc_scalar(J + DQ - 1, J)                                   # read two steps ago into buffer J % 2
+    desc_read(J)                                                 # op i + DQ + 1
     b_reads(J + PB, J + PB)
     a_load(J + AHEAD, J + AHEAD, f"s{J}")
     emit(f"s_cmp_lt_u32 s{S_AGE}, {AHEAD}")
@@ -238,14 +271,13 @@ emit("v_cmp_ne_u32 vcc, 0, %[sel01]")
 emit(f"v_mov_b32 v{V_AZB}, 0x80000000")
 emit(f"v_cndmask_b32 v{V_AZH}, %[a_voff], v{V_AZB}, vcc")
 emit(f"v_cndmask_b32 v{V_AZL}, v{V_AZB}, %[a_voff], vcc")
-# descriptors of ops 0 .. 4 into the ring
+# descriptors of ops 0 .. DQ - 2 into the ring
 for x in range(DQ - 1):
     emit(f"s_add_u32 s{S_T0}, %[win_lds], {16 * x}")
     emit(f"v_mov_b32 v{V_T0}, s{S_T0}")
     emit(f"ds_read_b128 v[{V_DESC}:{V_DESC + 3}], v{V_T0}")
     emit("s_waitcnt lgkmcnt(0)")
-    desc_scalar(x)
-emit(f"s_mov_b32 s{S_DP}, {16 * (DQ - 1)}")                        # op 5 is read below, made scalar in step 0
+    desc_scalar(x, 0)
 for x in range(AHEAD):
     a_load(x, x, f"p{x}")
 # copies of chunk 2, after the first A loads like the copies of a boundary
@@ -263,17 +295,19 @@ for it in range(4):
     emit(f"s_cbranch_scc0 Lpskip{it}_%=")
     emit(f"s_mov_b32 m0, s{S_T1}")
     emit("s_nop 0")
-    emit(f"global_load_lds_dwordx4 v{V_COPY}, %[sb{it}]")
-    emit(f"s_add_u32 s{S_BURST}, s{S_BURST}, 1")
+    if "copy" not in ABL:
+        emit(f"global_load_lds_dwordx4 v{V_COPY}, %[sb{it}]")
+        emit(f"s_add_u32 s{S_BURST}, s{S_BURST}, 1")
     label(f"Lpskip{it}")
     if it < 3:
         emit(f"s_add_u32 s{S_T1}, s{S_T1}, 1024")
 label("Lpnocopy")
-# LDS reads in flight when step 0 starts, oldest first, as in the steady state: descriptor of op 5, B of op 0, B of op 1
-emit(f"s_add_u32 s{S_T0}, s{S_DP}, %[win_lds]")
-emit(f"v_mov_b32 v{V_T0}, s{S_T0}")
-emit(f"ds_read_b128 v[{V_DESC}:{V_DESC + 3}], v{V_T0}")
+# LDS reads in flight when step 0 starts, oldest first, as in the steady state: descriptor of op DQ - 1 (buffer 0,
+# made scalar in step 0), B of op 0, descriptor of op DQ (buffer 1, made scalar in step 1), B of op 1
+emit(f"s_mov_b32 s{S_DP}, {16 * (DQ - 2)}")
+desc_read(0)
 b_reads(0, 0)
+desc_read(1)
 b_reads(1, 1)
 emit("s_branch Lstep_0_%=")
 
@@ -288,7 +322,7 @@ for x in range(AHEAD):
 label("Lexit")
 emit("s_waitcnt vmcnt(0) lgkmcnt(0)")
 
-clobber_v = [f"v{r}" for r in range(40, 128)]
+clobber_v = [f"v{r}" for r in range(V_FIRST, V_TOP)]
 clobber_s = [f"s{r}" for r in range(40, RING0 + 4 * UNROLL)]
 print("// Generated by gen_sweep_loop.py -- do not edit.")
 print("asm volatile(")

@@ -82,6 +82,7 @@ struct SweepArgs {
     const int32_t *chunk_ids;    // device: the K chunks in which the row group has blocks, ascending
     const int32_t *op_ptr;       // device, n_rg * SWEEP_WAVES + 1: range of (row group, wavefront) in ops
     const SweepOp *ops;          // device, op streams, SWEEP_OP_PAD slots of padding at the end
+    const int32_t *row_map;      // device, n_rg * SWEEP_G: block row of (row group, wavefront, local row), -1 = none
     int n_rg;
 };
 

@@ -9,7 +9,8 @@
 //    index is XOR-ed with a 4-bit function of n so that the 16 lanes of one ds_read_b128 phase
 //    (16 different n, same logical slot) hit 16 different 16-byte bank groups and the 16 lanes that
 //    fill one n write 256 contiguous bytes: no bank conflicts on either side.
-//  * Work.  A wavefront owns 8 block rows x 64 columns (128 fp32 accumulator registers) and runs a
+//  * Work.  A wavefront owns 8 of the 64 block rows (the plan picks which, so that the wavefronts have
+//    about the same work in every chunk) x 64 columns, 128 fp32 accumulator registers, and runs a
 //    host-built stream of ops.  One op = two blocks of one block row = one K = 32 step of
 //    v_mfma_f32_16x16x32_f16 per 16 columns (4 MFMAs).  The two blocks may sit in the same chunk or
 //    in two consecutive chunks (the ring keeps the previous stage), so few blocks stay unpaired; an
@@ -108,7 +109,7 @@ template <bool C_F32>
 __global__ __launch_bounds__(THREADS) void spmm_sweep_kernel(
     const uint16_t *__restrict__ vals, const uint16_t *__restrict__ B, void *__restrict__ Cout,
     const int32_t *__restrict__ rg_chunk_ptr, const int32_t *__restrict__ chunk_ids,
-    const int32_t *__restrict__ op_ptr, const SweepOp *__restrict__ ops, int Mb, int N, long K, int n_rg, int n_panels,
+    const int32_t *__restrict__ op_ptr, const SweepOp *__restrict__ ops, const int32_t *__restrict__ row_map, int N, long K, int n_rg, int n_panels,
     uint32_t vals_bytes)
 {
     extern __shared__ __align__(16) unsigned char lds[];
@@ -208,15 +209,18 @@ __global__ __launch_bounds__(THREADS) void spmm_sweep_kernel(
         const uint32_t sel01 = (uint32_t)sel;
         const uint32_t n_ops_u = __builtin_amdgcn_readfirstlane((uint32_t)n_ops), n_chunks_u = __builtin_amdgcn_readfirstlane((uint32_t)n_chunks);
         const uint32_t op_lo = (uint32_t)(uintptr_t)op_base, op_hi = (uint32_t)((uintptr_t)op_base >> 32);
-#include "spmm_sweep_loop.inc"
+#ifndef SWEEP_LOOP_INC
+#define SWEEP_LOOP_INC "spmm_sweep_loop.inc"
+#endif
+#include SWEEP_LOOP_INC
     }
     asm volatile("s_nop 15\n\ts_nop 15" ::: "memory"); // the last MFMAs retire before their results are read
 
     // Epilogue: tile (r, t), element e = C[(rg*64 + wave*8 + r)*16 + i16][n0 + 16*g + 4*t + e]
     auto store_row = [&](auto rc) {
         constexpr int R = decltype(rc)::value;
-        const int br = rg * SWEEP_G + wave * RW + R;
-        if (br >= Mb) return;
+        const int br = row_map[(rg * W + wave) * RW + R]; // the plan spreads the block rows of the group over the wavefronts
+        if (br < 0) return;
         const long m = (long)br * 16 + i16;
         const int nbase = n0 + 16 * g;
         const f32x4 v0 = read_acc<R, 0>(), v1 = read_acc<R, 1>(), v2 = read_acc<R, 2>(), v3 = read_acc<R, 3>();
@@ -259,11 +263,11 @@ hipError_t launch_sweep(const SweepArgs &a, hipStream_t st)
     dim3 grid((unsigned)wgs), block(THREADS);
     if (a.c_f32)
         hipLaunchKernelGGL((spmm_sweep_kernel<true>), grid, block, lds_bytes, st, a.vals, a.B, a.C,
-                           a.rg_chunk_ptr, a.chunk_ids, a.op_ptr, a.ops, (int)(a.M / 16), (int)a.N, (long)a.K,
+                           a.rg_chunk_ptr, a.chunk_ids, a.op_ptr, a.ops, a.row_map, (int)a.N, (long)a.K,
                            a.n_rg, n_panels, (uint32_t)(a.nnzb * 512));
     else
         hipLaunchKernelGGL((spmm_sweep_kernel<false>), grid, block, lds_bytes, st, a.vals, a.B, a.C,
-                           a.rg_chunk_ptr, a.chunk_ids, a.op_ptr, a.ops, (int)(a.M / 16), (int)a.N, (long)a.K,
+                           a.rg_chunk_ptr, a.chunk_ids, a.op_ptr, a.ops, a.row_map, (int)a.N, (long)a.K,
                            a.n_rg, n_panels, (uint32_t)(a.nnzb * 512));
     return hipGetLastError();
 }

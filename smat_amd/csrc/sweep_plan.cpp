@@ -31,9 +31,13 @@ void build_sweep_plan(const int32_t *row_ptr, const int32_t *col_idx, size_t mb,
     out = SweepPlanHost();
     out.rg_chunk_ptr.assign(n_rg + 1, 0);
     out.op_ptr.reserve(n_rg * WAVES + 1);
+    out.row_map.assign(n_rg * G, -1);
     std::vector<int32_t> local(n_kchunks, -1); // K chunk -> position in the row group's chunk list
+    struct RowOp { int32_t exec; SweepOpHost op; };
+    std::vector<RowOp> row_ops[G];
     struct Ranked { int rank; int row; SweepOpHost op; };
     std::vector<std::vector<Ranked>> by_chunk;
+    std::vector<int32_t> count; // ops of (row, chunk)
     for (size_t rg = 0; rg < n_rg; rg++) {
         const size_t r_begin = rg * G, r_end = std::min(mb, (rg + 1) * G);
         // the chunks this row group touches, ascending
@@ -46,52 +50,111 @@ void build_sweep_plan(const int32_t *row_ptr, const int32_t *col_idx, size_t mb,
             }
         const size_t n_chunks = out.chunk_ids.size() - first_chunk;
         out.rg_chunk_ptr[rg + 1] = (int32_t)out.chunk_ids.size();
+
+        // ---- ops of every block row: neighbouring blocks in pairs; w3 gets the local row later ----
+        count.assign((size_t)G * std::max<size_t>(n_chunks, 1), 0);
+        for (int lr = 0; lr < G; lr++) {
+            row_ops[lr].clear();
+            const size_t br = r_begin + (size_t)lr;
+            if (br >= r_end) continue;
+            int32_t q = row_ptr[br];
+            const int32_t q_end = row_ptr[br + 1];
+            while (q < q_end) {
+                const int32_t bc0 = col_idx[q] / 16;
+                const int32_t cl0 = local[(size_t)bc0 / S];
+                const uint32_t off0 = lds_offset(cl0, bc0 % S);
+                SweepOpHost op{0, off0, 0, 0};
+                int32_t exec = cl0;
+                bool pair = false;
+                if (q + 1 < q_end) {
+                    const int32_t bc1 = col_idx[q + 1] / 16;
+                    const int32_t cl1 = local[(size_t)bc1 / S];
+                    if (cl1 - cl0 <= 1) { // same chunk or the next listed one: both stages are resident
+                        op.w0 = (uint32_t)q * 512u;
+                        op.w2 = lds_offset(cl1, bc1 % S) - off0;
+                        exec = cl1;
+                        pair = true;
+                    }
+                }
+                if (!pair) { // both halves read the rows of B under this block; the missing half gets zeros of A
+                    if (q + 1 < nnzb) { // blocks (q, q + 1), the second multiplied by zeros
+                        op.w0 = (uint32_t)q * 512u;
+                        op.w3 = OP_ZERO_HI;
+                    } else { // last block of the matrix: blocks (q - 1, q), the first multiplied by zeros
+                        op.w0 = (uint32_t)(q - 1) * 512u;
+                        op.w3 = OP_ZERO_LO;
+                    }
+                }
+                (pair ? out.n_pairs : out.n_singles)++;
+                row_ops[lr].push_back(RowOp{exec, op});
+                count[(size_t)lr * n_chunks + (size_t)exec]++;
+                q += pair ? 2 : 1;
+            }
+        }
+
+        // ---- block rows -> wavefronts.  All wavefronts meet at a barrier once per chunk, so the cost of a chunk
+        // is the op count of its busiest wavefront: start from the block rows in order, then swap pairs of rows
+        // between wavefronts while the sum over chunks of that maximum falls (deterministic, a few passes). ----
+        int wave_of[G];
+        for (int lr = 0; lr < G; lr++) wave_of[lr] = lr / RW;
+        if (n_chunks > 0) {
+            std::vector<int32_t> load((size_t)WAVES * n_chunks, 0);
+            for (int lr = 0; lr < G; lr++)
+                for (size_t c = 0; c < n_chunks; c++) load[(size_t)wave_of[lr] * n_chunks + c] += count[(size_t)lr * n_chunks + c];
+            auto chunk_cost = [&](size_t c) {
+                int32_t m = MIN_OPS;
+                for (int w = 0; w < WAVES; w++) m = std::max(m, load[(size_t)w * n_chunks + c]);
+                return m;
+            };
+            for (int pass = 0; pass < 4; pass++) {
+                bool improved = false;
+                for (int i = 0; i < G; i++)
+                    for (int j = i + 1; j < G; j++) {
+                        const int wi = wave_of[i], wj = wave_of[j];
+                        if (wi == wj) continue;
+                        long delta = 0;
+                        for (size_t c = 0; c < n_chunks; c++) {
+                            const int32_t d = count[(size_t)j * n_chunks + c] - count[(size_t)i * n_chunks + c];
+                            if (d == 0) continue;
+                            const int32_t before = chunk_cost(c);
+                            load[(size_t)wi * n_chunks + c] += d;
+                            load[(size_t)wj * n_chunks + c] -= d;
+                            delta += chunk_cost(c) - before;
+                            load[(size_t)wi * n_chunks + c] -= d;
+                            load[(size_t)wj * n_chunks + c] += d;
+                        }
+                        if (delta < 0) {
+                            for (size_t c = 0; c < n_chunks; c++) {
+                                const int32_t d = count[(size_t)j * n_chunks + c] - count[(size_t)i * n_chunks + c];
+                                load[(size_t)wi * n_chunks + c] += d;
+                                load[(size_t)wj * n_chunks + c] -= d;
+                            }
+                            std::swap(wave_of[i], wave_of[j]);
+                            improved = true;
+                        }
+                    }
+                if (!improved) break;
+            }
+        }
+
+        // ---- op streams ----
         for (int w = 0; w < WAVES; w++) {
             out.op_ptr.push_back((int32_t)out.ops.size());
             by_chunk.assign(n_chunks, {});
-            for (int r = 0; r < RW; r++) {
-                const size_t br = r_begin + (size_t)w * RW + r;
-                if (br >= r_end) break;
-                int32_t q = row_ptr[br];
-                const int32_t q_end = row_ptr[br + 1];
-                while (q < q_end) {
-                    const int32_t bc0 = col_idx[q] / 16;
-                    const int32_t cl0 = local[(size_t)bc0 / S];
-                    const uint32_t off0 = lds_offset(cl0, bc0 % S);
-                    SweepOpHost op{0, 0, 0, 0};
-                    int32_t exec = cl0;
-                    bool pair = false;
-                    if (q + 1 < q_end) {
-                        const int32_t bc1 = col_idx[q + 1] / 16;
-                        const int32_t cl1 = local[(size_t)bc1 / S];
-                        if (cl1 - cl0 <= 1) { // same chunk or the next listed one: both stages are resident
-                            op.w0 = (uint32_t)q * 512u;
-                            op.w1 = off0;
-                            op.w2 = lds_offset(cl1, bc1 % S) - off0;
-                            op.w3 = (uint32_t)r * ROW_CODE << 23;
-                            exec = cl1;
-                            pair = true;
-                        }
-                    }
-                    if (!pair) {
-                        if (q + 1 < nnzb) { // blocks (q, q + 1), the second multiplied by zeros
-                            op.w0 = (uint32_t)q * 512u;
-                            op.w3 = OP_ZERO_HI | ((uint32_t)r * ROW_CODE << 23);
-                        } else { // last block of the matrix: blocks (q - 1, q), the first multiplied by zeros
-                            op.w0 = (uint32_t)(q - 1) * 512u;
-                            op.w3 = OP_ZERO_LO | ((uint32_t)r * ROW_CODE << 23);
-                        }
-                        op.w1 = off0; // both halves read the rows of B under this block
-                        op.w2 = 0;
-                    }
-                    (pair ? out.n_pairs : out.n_singles)++;
+            int r = 0;
+            for (int lr = 0; lr < G; lr++) {
+                if (wave_of[lr] != w) continue;
+                if (r_begin + (size_t)lr < r_end) out.row_map[(rg * WAVES + (size_t)w) * RW + (size_t)r] = (int32_t)(r_begin + (size_t)lr);
+                for (const RowOp &ro : row_ops[lr]) {
+                    SweepOpHost op = ro.op;
+                    op.w3 |= (uint32_t)r * ROW_CODE << 23;
                     // rank = how many ops of this block row the chunk already holds: ops of one block
                     // row (same accumulators) end up spread over the chunk
                     int rank = 0;
-                    for (const Ranked &x : by_chunk[(size_t)exec]) rank += x.row == r;
-                    by_chunk[(size_t)exec].push_back(Ranked{rank, r, op});
-                    q += pair ? 2 : 1;
+                    for (const Ranked &x : by_chunk[(size_t)ro.exec]) rank += x.row == r;
+                    by_chunk[(size_t)ro.exec].push_back(Ranked{rank, r, op});
                 }
+                r++;
             }
             for (size_t c = 0; c < n_chunks; c++) {
                 std::vector<Ranked> &list = by_chunk[c];
@@ -118,13 +181,13 @@ void build_sweep_plan(const int32_t *row_ptr, const int32_t *col_idx, size_t mb,
 } // namespace smat
 
 // Test hook (not part of smat.h): builds the work list on the host and hands it out.  Arrays are
-// allocated with malloc; release each with smat_host_free.  counts[0..5] = row groups, listed
+// allocated with malloc; release each with smat_host_free.  row_map: n_rg * 64 block rows (-1 = none).  counts[0..5] = row groups, listed
 // chunks, ops (with fillers, without padding), pairs, singles, fillers.
 extern "C" int smat_internal_sweep_plan(const int32_t *row_ptr, const int32_t *col_idx, size_t M, size_t K,
                                          int32_t **rg_chunk_ptr, int32_t **chunk_ids, int32_t **op_ptr,
-                                         uint32_t **ops, int64_t *counts)
+                                         uint32_t **ops, int32_t **row_map, int64_t *counts)
 {
-    if (!row_ptr || !col_idx || !rg_chunk_ptr || !chunk_ids || !op_ptr || !ops || !counts) return SMAT_ERR_INVALID;
+    if (!row_ptr || !col_idx || !rg_chunk_ptr || !chunk_ids || !op_ptr || !ops || !row_map || !counts) return SMAT_ERR_INVALID;
     if (M == 0 || M % 16 || K % 16 || row_ptr[M / 16] < 2) return SMAT_ERR_INVALID;
     smat::SweepPlanHost p;
     try {
@@ -141,7 +204,8 @@ extern "C" int smat_internal_sweep_plan(const int32_t *row_ptr, const int32_t *c
     *chunk_ids = (int32_t *)dup(p.chunk_ids.data(), p.chunk_ids.size() * 4);
     *op_ptr = (int32_t *)dup(p.op_ptr.data(), p.op_ptr.size() * 4);
     *ops = (uint32_t *)dup(p.ops.data(), p.ops.size() * 16);
-    if (!*rg_chunk_ptr || !*chunk_ids || !*op_ptr || !*ops) return SMAT_ERR_NOMEM;
+    *row_map = (int32_t *)dup(p.row_map.data(), p.row_map.size() * 4);
+    if (!*rg_chunk_ptr || !*chunk_ids || !*op_ptr || !*ops || !*row_map) return SMAT_ERR_NOMEM;
     counts[0] = (int64_t)p.rg_chunk_ptr.size() - 1;
     counts[1] = (int64_t)p.chunk_ids.size();
     counts[2] = (int64_t)p.ops.size() - 384;

@@ -17,6 +17,7 @@ struct SweepPlanHost {
     std::vector<int32_t> rg_chunk_ptr; // n_rg + 1
     std::vector<int32_t> chunk_ids;    // K chunk of every (row group, listed chunk)
     std::vector<int32_t> op_ptr;       // n_rg * 8 + 1
+    std::vector<int32_t> row_map;      // n_rg * 64: block row of (row group, wavefront, local row), -1 = none
     std::vector<SweepOpHost> ops;      // op streams + padding
     size_t n_pairs = 0, n_singles = 0, n_fillers = 0;
 };

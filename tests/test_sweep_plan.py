@@ -21,10 +21,10 @@ PAD = 384
 def sweep_plan(row_ptr, col_idx, M, K):
     fn = lib.smat_internal_sweep_plan
     fn.restype = C.c_int
-    fn.argtypes = [C.c_void_p, C.c_void_p, C.c_size_t, C.c_size_t] + [C.POINTER(C.c_void_p)] * 4 + [C.POINTER(C.c_int64)]
+    fn.argtypes = [C.c_void_p, C.c_void_p, C.c_size_t, C.c_size_t] + [C.POINTER(C.c_void_p)] * 5 + [C.POINTER(C.c_int64)]
     row_ptr = np.ascontiguousarray(row_ptr, np.int32)
     col_idx = np.ascontiguousarray(col_idx, np.int32)
-    out = [C.c_void_p() for _ in range(4)]
+    out = [C.c_void_p() for _ in range(5)]
     counts = (C.c_int64 * 6)()
     rc = fn(row_ptr.ctypes.data, col_idx.ctypes.data, M, K, *[C.byref(o) for o in out], counts)
     assert rc == 0
@@ -37,6 +37,7 @@ def sweep_plan(row_ptr, col_idx, M, K):
     return {
         "rg_chunk_ptr": take(out[0], n_rg + 1, np.int32), "chunk_ids": take(out[1], n_chunks, np.int32),
         "op_ptr": take(out[2], n_rg * WAVES + 1, np.int32), "ops": take(out[3], (n_ops + PAD) * 4, np.uint32).reshape(-1, 4),
+        "row_map": take(out[4], n_rg * G, np.int32),
         "pairs": counts[3], "singles": counts[4], "fillers": counts[5], "n_ops": n_ops,
     }
 
@@ -76,7 +77,9 @@ def replay(plan, A, Bd):
                 assert (int(w3) >> 23) % 40 == 0
                 r = (int(w3) >> 23) // 40
                 assert r < RW
-                br = rg * G + w * RW + r
+                br = int(plan["row_map"][(rg * WAVES + w) * RW + r])
+                if int(w3) & (ZERO_HI | ZERO_LO) != (ZERO_HI | ZERO_LO):  # a filler may sit in a wavefront without rows
+                    assert 0 <= br < M // 16 and br // G == rg
                 off1 = (int(w1) + int(np.int32(w2))) & 0xFFFFFFFF
                 for half, (off, zero) in enumerate(((int(w1), w3 & ZERO_LO), (off1, w3 & ZERO_HI))):
                     stage, slab = slot_of(off)
@@ -93,6 +96,8 @@ def replay(plan, A, Bd):
                     Cd[br * 16:br * 16 + 16] += blocks[blk] @ Bd[k0:k0 + 16]
             assert cur == chunks.size - 1 and in_chunk >= 2
     assert np.all(used == 1), "a block is multiplied zero or several times"
+    rows = plan["row_map"][plan["row_map"] >= 0]
+    assert np.array_equal(np.sort(rows), np.arange(M // 16)), "row_map is not a partition of the block rows"
     # read-ahead: the descriptors after the last op exist and are harmless
     tail = plan["ops"][plan["n_ops"]:]
     assert tail.shape[0] == PAD and np.all(tail[:, :3] == 0) and np.all(tail[:, 3] == (ZERO_HI | ZERO_LO))
