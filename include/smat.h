@@ -127,6 +127,21 @@ int smat_spmm_bcsr_f16_ex(const uint16_t *vals, const int32_t *row_ptr, const in
                           const uint16_t *B, void *C, size_t M, size_t N, size_t K, size_t nnzb,
                           const smat_spmm_opts *opts, const smat_plan *plan);
 
+/* ---- SpMM that allocates nothing ------------------------------------------
+ * No counterpart in the reference.  For callers that cannot allocate device memory: code under HIP graph
+ * capture, tight serving loops, harnesses that forbid hipMalloc.  Same operands and result type as
+ * smat_spmm_bcsr_f16 plus the stream.  It runs what a SMAT_KERNEL_ROWWISE_PACKED plan runs for whole block
+ * rows (B is first repacked slab-major, then the row-wise kernel), with the copy of B in a fixed array inside
+ * the library instead of plan-owned memory: it calls no hipMalloc / hipFree.
+ * Limit: K * N * 2 <= SMAT_STATIC_SCRATCH_BYTES, else SMAT_ERR_UNSUPPORTED.  Each GPU the library runs on holds
+ * one such array until the process ends.  Every call on a GPU uses that GPU's array: calls that overlap on one
+ * GPU (two streams, two threads) race; calls on one stream are ordered.  Nothing in the array has to survive
+ * between calls (the repack rewrites every element it reads). */
+#define SMAT_STATIC_SCRATCH_BYTES (64u << 20)
+int smat_spmm_bcsr_f16_static(const uint16_t *vals, const int32_t *row_ptr, const int32_t *col_idx,
+                              const uint16_t *B, uint16_t *C, size_t M, size_t N, size_t K, size_t nnzb,
+                              void *stream);
+
 /* ---- matrix load: Matrix Market -> CSR (host) ----------------------------
  * Replaces mmio_allinone (src/cuda_hgemm/src/common/mmio_highlevel.h:619-786):
  * M and K come back rounded up to multiples of 16, symmetric/hermitian files

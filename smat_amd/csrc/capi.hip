@@ -162,6 +162,53 @@ extern "C" int smat_spmm_bcsr_f16(const uint16_t *vals, const int32_t *row_ptr,
     return smat_spmm_bcsr_f16_ex(vals, row_ptr, col_idx, B, C, M, N, K, nnzb, nullptr, nullptr);
 }
 
+// ---- SpMM without any allocation ------------------------------------------------
+// For callers that cannot allocate (HIP graph capture, serving loops, harnesses that forbid hipMalloc): the
+// row-wise kernel on a slab-major copy of B, like a SMAT_KERNEL_ROWWISE_PACKED plan, with the copy in a
+// fixed array of the library instead of plan-owned memory.  One array per GPU, held until the process ends.
+static __device__ __align__(256) unsigned char scratch[SMAT_STATIC_SCRATCH_BYTES];
+
+#include <mutex>
+namespace {
+constexpr int MAX_DEVICES = 64;
+std::mutex g_scratch_mutex;
+void *g_scratch_ptr[MAX_DEVICES] = {nullptr}; // device address of `scratch` on each GPU (the name is no device address)
+} // namespace
+
+extern "C" int smat_spmm_bcsr_f16_static(const uint16_t *vals, const int32_t *row_ptr, const int32_t *col_idx,
+                                          const uint16_t *B, uint16_t *C, size_t M, size_t N, size_t K, size_t nnzb,
+                                          void *stream)
+{
+    int rc = check_shapes(vals, row_ptr, col_idx, B, C, M, N, K, nnzb);
+    if (rc) return rc;
+    if (K * N * sizeof(uint16_t) > (size_t)SMAT_STATIC_SCRATCH_BYTES || K * N / N != K)
+        return set_error(SMAT_ERR_UNSUPPORTED,
+                         "smat_spmm_bcsr_f16_static: B (%zu x %zu fp16) exceeds the fixed scratch of %zu bytes", K, N,
+                         (size_t)SMAT_STATIC_SCRATCH_BYTES);
+    int dev = 0;
+    SMAT_HIP(hipGetDevice(&dev));
+    if (dev < 0 || dev >= MAX_DEVICES) return set_error(SMAT_ERR_UNSUPPORTED, "device ordinal %d out of range", dev);
+    void *ptr;
+    {
+        std::lock_guard<std::mutex> lock(g_scratch_mutex);
+        if (!g_scratch_ptr[dev]) { // once per device, with that device current
+            void *p = nullptr;
+            SMAT_HIP(hipGetSymbolAddress(&p, HIP_SYMBOL(scratch)));
+            g_scratch_ptr[dev] = p;
+        }
+        ptr = g_scratch_ptr[dev];
+    }
+    SpmmArgs a{};
+    a.vals = vals; a.row_ptr = row_ptr; a.col_idx = col_idx; a.B = B; a.C = C;
+    a.M = M; a.N = N; a.K = K; a.nnzb = nnzb;
+    a.c_f32 = false;
+    a.n_items = (int)(M / 16); // whole block rows, one wavefront each: no work list, no partial tiles
+    a.b_packed = static_cast<uint16_t *>(ptr); // every element the kernel reads is rewritten by the repack first
+    hipError_t e = launch_rowwise(a, static_cast<hipStream_t>(stream));
+    if (e != hipSuccess) return set_error(SMAT_ERR_HIP, "SpMM launch failed: %s", hipGetErrorString(e));
+    return SMAT_OK;
+}
+
 // ---- plans -----------------------------------------------------------------
 
 extern "C" int smat_plan_create(smat_plan **out, const int32_t *row_ptr_host,
