@@ -27,25 +27,55 @@ sys.path.insert(0, ROOT)
 PEAK_FP16_TFLOPS = 2500.0  # MI355X dense fp16 MFMA
 PEAK_HBM_GBS = 8000.0      # MI355X HBM3E
 
-# HBM bytes per launch measured with rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE and scaled by a plain
-# device copy of known size (summaries under profiles/): (workload, kernel id) -> bytes
-MEASURED_TRAFFIC = {
-    ("block_pruned_8192_10pct_N4096", 2): 143469 * 1024 * 2.0 + 66082 * 1024 * 1.0,
-    # row-wise kernel + repack kernel
-    ("block_pruned_8192_10pct_N4096", 1): (247966 + 32783) * 1024 * 2.0 + (65538 + 65536) * 1024 * 1.0,
-    # compact kernel + transpose kernel (+ reduce kernel for the split rows of R-MAT)
-    ("er_16384_0.1pct_reordered_N256", 5): (25992 + 4111) * 1024 * 2.0 + (8192 + 8192) * 1024 * 1.0,
-    ("rmat_s20_deg16_N128", 5): (1531955 + 131089 + 37914) * 1024 * 2.0 + (327815 + 262144 + 10068) * 1024 * 1.0,
-    ("stencil27_64_N64", 5): (70391 + 16399) * 1024 * 2.0 + (32768 + 32768) * 1024 * 1.0,
-}
+KERNEL_NAMES = {1: "rowwise", 2: "sweep", 3: "rowwise", 5: "compact"}
 
 
-# Share of SIMD cycles with the MFMA pipe busy, rocprofv3 --pmc SQ_VALU_MFMA_BUSY_CYCLES / SQ_BUSY_CYCLES
-# (same summaries): informational, next to the roofline fraction
-MEASURED_MFMA_BUSY = {
-    ("block_pruned_8192_10pct_N4096", 2): 0.217,
-    ("block_pruned_8192_10pct_N4096", 1): 0.168,
-}
+def profiled(workload, kernel_id):
+    """HBM traffic per launch (bytes) and MFMA-busy share that rocprofv3 counted for this kernel on this
+    workload, read from the committed summary profiles/spmm_<kernel>_<workload>.md (lines
+    `traffic_bytes_per_launch: <number>` and `mfma_busy: <number>`), with the file as `source`.
+    Nothing is returned for a pair that has no summary: counters are never measured inside this run."""
+    import re
+    path = os.path.join(ROOT, "profiles", f"spmm_{KERNEL_NAMES.get(kernel_id, kernel_id)}_{workload}.md")
+    if not os.path.exists(path):
+        return {}
+    text = open(path).read()
+    out = {}
+    for key in ("traffic_bytes_per_launch", "mfma_busy"):
+        m = re.search(rf"^{key}:\s*([0-9.eE+]+)", text, re.M)
+        if m:
+            out[key] = float(m.group(1))
+    if out:
+        out["source"] = os.path.relpath(path, ROOT)
+    return out
+
+
+def sha256_of(*arrays):
+    import hashlib
+    h = hashlib.sha256()
+    for a in arrays:
+        h.update(np.ascontiguousarray(a).tobytes())
+    return h.hexdigest()
+
+
+def verify_sample(A, B, N, C_bits, n_sample=24, tol=1e-3):
+    """The result of the last timed launch against the CPU oracle on block rows spread over the matrix
+    (first, last, and evenly spaced ones between).  Returns the worst error relative to the row L2 norm;
+    the caller fails the run above `tol` (fp16 output of an fp32-accumulated product)."""
+    from tests.oracle_lib import load_oracle
+    oracle = load_oracle()
+    rp, ci = A["b_row_ptr"], A["b_col_idx"]
+    mb = A["M"] // 16
+    rows = np.unique(np.linspace(0, mb - 1, min(mb, n_sample)).astype(np.int64))
+    keep = np.concatenate([np.arange(rp[r], rp[r + 1]) for r in rows]).astype(np.int64)
+    sub_rp = np.concatenate([[0], np.cumsum([rp[r + 1] - rp[r] for r in rows])]).astype(np.int32)
+    want = oracle.spmm_bcsr(16 * rows.size, N, A["K"], sub_rp, ci[keep], A["b_val"].reshape(-1, 256)[keep].ravel(), B,
+                            threads=max(1, min(16, os.cpu_count() or 1, oracle.max_threads())))
+    got = np.concatenate([C_bits[16 * r:16 * r + 16] for r in rows])
+    rel, max_abs, _ = oracle.compare(got, want)
+    return {"block_rows": int(rows.size), "blocks": int(keep.size), "max_rel_to_row_l2": float(f"{rel:.3e}"),
+            "max_abs": float(f"{max_abs:.3e}"), "tolerance": tol, "ok": bool(rel <= tol and np.isfinite(rel))}
+
 
 INFO = {}  # facts about the generated workload that go into the config of the result line
 PERM_FILE = None
@@ -70,6 +100,7 @@ def build_workload(name):
             pr, pc, _, _ = smat_amd.reorder_csr(d["M"], d["K"], d["row_ptr"], d["col_idx"], 16, 16, 0.5, True)
             INFO["reorder_s"] = round(time.perf_counter() - t0, 3)
             INFO["nnzb_before_reorder"] = int(b.nnzb)
+            INFO["perm_sha256"] = sha256_of(np.asarray(pr, np.int64), np.asarray(pc, np.int64))
             rp, ci, v = smat_amd.permute_csr(d["M"], d["K"], d["row_ptr"], d["col_idx"], d["val"], pr, pc)
             b = smat_amd.csr_to_bcsr(d["M"], d["K"], rp, ci, v)
         A = {"M": b.M, "K": b.K, "b_row_ptr": b.row_ptr, "b_col_idx": b.col_idx, "b_val": b.val, "nnzb": b.nnzb}
@@ -83,6 +114,7 @@ def build_workload(name):
             pr, pc, _, _ = smat_amd.reorder_csr(d["M"], d["K"], d["row_ptr"], d["col_idx"], 16, 16, 0.5, True)
             INFO["reorder_s"] = round(time.perf_counter() - t0, 3)
             INFO["nnzb_before_reorder"] = int(b.nnzb)
+            INFO["perm_sha256"] = sha256_of(np.asarray(pr, np.int64), np.asarray(pc, np.int64))
             rp, ci, v = smat_amd.permute_csr(d["M"], d["K"], d["row_ptr"], d["col_idx"], d["val"], pr, pc)
             b = smat_amd.csr_to_bcsr(d["M"], d["K"], rp, ci, v)
         A = {"M": b.M, "K": b.K, "b_row_ptr": b.row_ptr, "b_col_idx": b.col_idx, "b_val": b.val, "nnzb": b.nnzb}
@@ -98,6 +130,7 @@ def build_workload(name):
             z = np.load(PERM_FILE)
             INFO["reorder_s"] = float(z["reorder_s"])
             INFO["nnzb_before_reorder"] = int(b.nnzb)
+            INFO["perm_sha256"] = sha256_of(np.asarray(z["perm_rows"], np.int64), np.asarray(z["perm_cols"], np.int64))
             rp, ci, v = smat_amd.permute_csr(d["M"], d["K"], d["row_ptr"], d["col_idx"], d["val"],
                                              z["perm_rows"], z["perm_cols"])
             b = smat_amd.csr_to_bcsr(d["M"], d["K"], rp, ci, v)
@@ -197,6 +230,7 @@ def main():
     ap.add_argument("--kernel", type=int, default=0, help="0 auto, 1 rowwise, 2 sweep, 3 rowwise reading B in place, 5 compact")
     ap.add_argument("--no-plan", action="store_true")
     ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--no-verify", action="store_true", help="skip the check of sampled block rows against the CPU oracle")
     ap.add_argument("--no-attach-values", action="store_true",
                     help="do not let the plan look at the block values (the compact kernel, id 5, needs them)")
     ap.add_argument("--perm-file", default=None, help="npz with perm_rows / perm_cols / reorder_s (reordered R-MAT workload)")
@@ -265,6 +299,34 @@ def main():
     lib.smat_event_destroy(ev0)
     lib.smat_event_destroy(ev1)
 
+    # every launch on its own: event pairs around single launches (the gaps between launches are not in them)
+    n_single = min(args.steps, 50)
+    pairs = []
+    for _ in range(n_single):
+        e0, e1 = C.c_void_p(), C.c_void_p()
+        check(lib.smat_event_create(C.byref(e0)))
+        check(lib.smat_event_create(C.byref(e1)))
+        check(lib.smat_event_record(e0, None))
+        step()
+        check(lib.smat_event_record(e1, None))
+        pairs.append((e0, e1))
+    torch.cuda.synchronize()
+    singles = []
+    for e0, e1 in pairs:
+        check(lib.smat_event_elapsed_ms(e0, e1, C.byref(ms)))
+        singles.append(ms.value)
+        lib.smat_event_destroy(e0)
+        lib.smat_event_destroy(e1)
+    singles = np.array(singles)
+
+    # the result of the last launch against the CPU oracle, before anything is reported
+    check_result = None
+    if not args.no_verify:
+        check_result = verify_sample(A, B, N, Cd.cpu().numpy().view(np.uint16))
+
+    peak = C.c_double()
+    check(lib.smat_bench_mfma_peak(C.byref(peak)))
+
     flops = 2.0 * nnzb * 256 * N
     qbytes = algorithmic_bytes(A, N)
     value = flops / (wall_ms * 1e-3) / 1e9
@@ -278,12 +340,20 @@ def main():
         roof = {"bound": "hbm", "achieved": round(ach_gbs, 1), "peak": PEAK_HBM_GBS, "unit": "GB/s",
                 "frac": round(ach_gbs / PEAK_HBM_GBS, 4)}
     kernel_id = (plan.info()["kernel"] if plan is not None else 1) if args.kernel == 0 else args.kernel
-    if kernel_id == 1 and (plan is None or not plan.info()["b_pack_bytes"]):
-        kernel_id = 3
-    roof["traffic"] = MEASURED_TRAFFIC.get((args.workload, kernel_id))
-    if (args.workload, kernel_id) in MEASURED_MFMA_BUSY:
-        roof["mfma_busy_rocprof"] = MEASURED_MFMA_BUSY[(args.workload, kernel_id)]
+    if kernel_id == 4:
+        kernel_id = 1
+    prof = profiled(args.workload, kernel_id)
+    roof["traffic"] = prof.get("traffic_bytes_per_launch")
+    if prof:
+        roof["profile_source"] = prof["source"]
+        if "mfma_busy" in prof:
+            roof["mfma_busy_rocprof"] = prof["mfma_busy"]
     roof["kernel_ms"] = round(kernel_ms, 5)
+    roof["kernel_ms_single_launch"] = {"n": int(singles.size), "median": round(float(np.median(singles)), 5),
+                                       "min": round(float(singles.min()), 5), "max": round(float(singles.max()), 5)}
+    roof["measured_mfma_peak_tflops"] = round(peak.value, 1)
+    if mfma_bound and peak.value > 0:
+        roof["frac_of_measured_mfma_peak"] = round(ach_tflops / peak.value, 4)
     roof["algorithmic_flops"] = flops
     roof["algorithmic_bytes"] = qbytes
     roof["hbm_gbs_at_algorithmic_bytes"] = round(ach_gbs, 1)
@@ -302,8 +372,10 @@ def main():
         "dtype": "f16",
         "data": "synthetic",
         "config": {"workload": args.workload, "M": M, "K": K, "N": N, "nnzb": nnzb, "block": 16,
-                   "c_dtype": "f16", "plan": None if plan is None else plan.info(), **INFO},
+                   "c_dtype": "f16", "plan": None if plan is None else plan.info(),
+                   "pattern_sha256": sha256_of(A["b_row_ptr"].astype(np.int32), A["b_col_idx"].astype(np.int32)), **INFO},
         "roofline": roof,
+        "verified": check_result,
     }
     if not args.no_cpu_baseline:
         port = cpu_baseline(A, B, N)
@@ -312,6 +384,8 @@ def main():
         if ref is not None:
             out["cpu_baseline_all_cores"] = port
     print(json.dumps(out))
+    if check_result is not None and not check_result["ok"]:
+        raise SystemExit(f"bench.py: the result of the last launch differs from the CPU oracle: {check_result}")
 
 
 if __name__ == "__main__":

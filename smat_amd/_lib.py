@@ -73,6 +73,7 @@ SIGNATURES = {
     "smat_event_record": (_int, [_vp, _vp]),
     "smat_event_synchronize": (_int, [_vp]),
     "smat_event_elapsed_ms": (_int, [_vp, _vp, C.POINTER(C.c_float)]),
+    "smat_bench_mfma_peak": (_int, [C.POINTER(C.c_double)]),
 }
 
 

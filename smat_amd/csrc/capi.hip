@@ -475,3 +475,58 @@ extern "C" int smat_event_elapsed_ms(void *a, void *b, float *ms)
     SMAT_HIP(hipEventElapsedTime(ms, (hipEvent_t)a, (hipEvent_t)b));
     return SMAT_OK;
 }
+
+// ---- what the MFMA pipes of this device deliver --------------------------------
+// A kernel of nothing but v_mfma_f32_16x16x32_f16 on registers: 8 wavefronts per workgroup, 8 independent
+// accumulators each, one workgroup per CU and launch slot.  The rate it reaches is the ceiling any fp16 kernel
+// on this device and clock can approach; benchmarks quote it next to the published peak.
+namespace {
+typedef _Float16 peak_f16x8 __attribute__((ext_vector_type(8)));
+typedef float peak_f32x4 __attribute__((ext_vector_type(4)));
+__global__ __launch_bounds__(512) void mfma_peak_kernel(float *out, int iters)
+{
+    peak_f32x4 acc[8];
+    for (int t = 0; t < 8; t++) acc[t] = (peak_f32x4){0, 0, 0, 0};
+    const _Float16 x = (_Float16)(0.001f * (threadIdx.x & 7)), y = (_Float16)(threadIdx.x & 3);
+    peak_f16x8 a = {x, x, x, x, x, x, x, x}, b = {y, y, y, y, y, y, y, y};
+    for (int i = 0; i < iters; i++) {
+#pragma unroll
+        for (int t = 0; t < 8; t++) acc[t] = __builtin_amdgcn_mfma_f32_16x16x32_f16(a, b, acc[t], 0, 0, 0);
+    }
+    float s = 0;
+    for (int t = 0; t < 8; t++) s += acc[t][0] + acc[t][1] + acc[t][2] + acc[t][3];
+    if (s == 12345.678f) out[0] = s; // keeps the loop alive, never true for these operands
+}
+} // namespace
+
+extern "C" int smat_bench_mfma_peak(double *tflops)
+{
+    if (!tflops) return set_error(SMAT_ERR_INVALID, "tflops must not be NULL");
+    hipDeviceProp_t prop;
+    int dev = 0;
+    SMAT_HIP(hipGetDevice(&dev));
+    SMAT_HIP(hipGetDeviceProperties(&prop, dev));
+    const int cus = prop.multiProcessorCount, iters = 16384;
+    float *out = nullptr;
+    SMAT_HIP(hipMalloc(&out, sizeof(float)));
+    hipEvent_t e0, e1;
+    SMAT_HIP(hipEventCreate(&e0));
+    SMAT_HIP(hipEventCreate(&e1));
+    double best = 0;
+    for (int rep = 0; rep < 4; rep++) { // first pass warms the clocks
+        SMAT_HIP(hipEventRecord(e0, nullptr));
+        hipLaunchKernelGGL(mfma_peak_kernel, dim3(cus), dim3(512), 0, nullptr, out, iters);
+        SMAT_HIP(hipEventRecord(e1, nullptr));
+        SMAT_HIP(hipEventSynchronize(e1));
+        float ms = 0;
+        SMAT_HIP(hipEventElapsedTime(&ms, e0, e1));
+        const double flops = (double)cus * 8 * iters * 8 * 2.0 * 16 * 16 * 32;
+        if (rep && ms > 0) best = std::max(best, flops / (ms * 1e-3) / 1e12);
+    }
+    (void)hipEventDestroy(e0);
+    (void)hipEventDestroy(e1);
+    (void)hipFree(out);
+    SMAT_HIP(hipGetLastError());
+    *tflops = best;
+    return SMAT_OK;
+}
