@@ -11,6 +11,10 @@ the input CSR pattern, the GROUPING line of `<out>.g`, the row order of
 `<case>_reordered.el`, and the integer statistics comparison_counter,
 merge_counter, VBR_nzblocks_count and VBR_longest_row from the stats file.
 Only data is stored; nothing of the reference's code.
+
+It also records the two-pass flow of src/reorder.py:107-182 into tests/golden/reorder_two_pass/*.npz:
+the program on <case>.el, then on the transpose of <case>_reordered.el ((u, v) -> (v, u), lines sorted,
+src/reorder.py:82-104), with both GROUPING lines, both reordered edge lists and both sets of counters.
 """
 import os
 import subprocess
@@ -115,6 +119,48 @@ def run_reference(r, c, col_block, row_block, tau, workdir):
                                          dtype=np.int64)
 
 
+TWO_PASS = {
+    # name: (case of CASES, col_block, row_block, tau)
+    "er_256": ("er_256", 16, 16, 0.5),
+    "er_rect_600x900": ("er_rect_600x900", 16, 16, 0.5),
+    "er_gaps_500": ("er_gaps_500", 16, 16, 0.5),
+    "stencil_8": ("stencil_8", 16, 16, 0.5),
+    "rmat_10": ("rmat_10", 16, 16, 0.5),
+    "clustered_800_b8": ("clustered_800", 8, 16, 0.5),
+}
+
+
+def run_two_pass(r, c, col_block, row_block, tau, workdir):
+    """Both runs of the reference program; returns per pass (grouping, reordered edge list, counters)."""
+    first = run_reference(r, c, col_block, row_block, tau, workdir)
+    reordered = first[1]
+    second_dir = os.path.join(workdir, "t")
+    os.makedirs(second_dir)
+    second = run_reference(reordered[:, 1], reordered[:, 0], col_block, row_block, tau, second_dir)  # write_el sorts the lines
+    return first, second
+
+
+def main_two_pass():
+    out_dir = os.path.join(HERE, "reorder_two_pass")
+    os.makedirs(out_dir, exist_ok=True)
+    for name, (case, cb, rb, tau) in TWO_PASS.items():
+        r, c = CASES[case][0]()
+        order = np.lexsort((c, r))
+        r, c = r[order], c[order]
+        rows = int(r.max()) + 1
+        row_ptr = np.zeros(rows + 1, dtype=np.int64)
+        np.add.at(row_ptr, r + 1, 1)
+        with tempfile.TemporaryDirectory() as wd:
+            (g1, el1, st1), (g2, el2, st2) = run_two_pass(r, c, cb, rb, tau, wd)
+        np.savez_compressed(os.path.join(out_dir, name + ".npz"), rows=np.int64(rows), cols=np.int64(c.max() + 1),
+                            row_ptr=np.cumsum(row_ptr).astype(np.int32), col_idx=c.astype(np.int32),
+                            params=np.array([cb, rb, tau], dtype=np.float64),
+                            grouping_rows=g1.astype(np.int32), grouping_cols=g2.astype(np.int32),
+                            row_pass_el=el1.astype(np.int32), col_pass_el=el2.astype(np.int32),
+                            stats_rows=st1, stats_cols=st2)
+        print(f"two-pass {name} b={cb} B={rb} tau={tau}: rows={rows} stats {st1.tolist()} then {st2.tolist()}")
+
+
 def main():
     if not os.path.exists(REF_BIN):
         sys.exit(f"{REF_BIN} missing: run `make -C oracle ref` first")
@@ -144,3 +190,4 @@ def main():
 
 if __name__ == "__main__":
     main()
+    main_two_pass()

@@ -1,0 +1,122 @@
+"""The benchmark configurations at their real sizes on the GPU: sampled block rows (the whole result where
+the CPU oracle finishes in seconds) against the oracle, plus properties that do not depend on the size.
+
+Bar as in test_gpu_spmm.py: max_j |C[i][j] - ref[i][j]| / ||ref[i][:]||_2 <= 1e-3 for the fp16 output."""
+import numpy as np
+import pytest
+
+from smat_amd import generators as gen
+from tests.test_gpu_spmm import TOL_F16, bcsr_of, gpu_spmm_compact, oracle_ref, to_dev
+
+pytestmark = pytest.mark.gpu
+
+
+def sample_rows(mb, n, extra=()):
+    return np.unique(np.concatenate([np.linspace(0, mb - 1, min(mb, n)).astype(np.int64), np.asarray(extra, np.int64)]))
+
+
+def check_sampled(oracle, A, B_bits, N, C_bits, rows):
+    """Block rows `rows` of the fp16 result C_bits (M x N, uint16) against the oracle on those rows alone."""
+    rp, ci = A["b_row_ptr"].astype(np.int64), A["b_col_idx"]
+    sel = np.concatenate([np.arange(rp[r], rp[r + 1]) for r in rows])
+    sub = {"M": 16 * len(rows), "K": A["K"],
+           "b_row_ptr": np.concatenate([[0], np.cumsum([rp[r + 1] - rp[r] for r in rows])]).astype(np.int32),
+           "b_col_idx": ci[sel], "b_val": A["b_val"].reshape(-1, 256)[sel].ravel()}
+    ref = oracle_ref(oracle, sub, B_bits, N)
+    got = np.concatenate([C_bits[16 * r:16 * r + 16] for r in rows])
+    err = oracle.compare(got, ref)[0]
+    assert err <= TOL_F16, err
+
+
+@pytest.mark.timeout(600)
+def test_config3_rmat_scale20_full_size(smat, cuda, oracle):
+    """R-MAT scale 20, average degree 16, N = 128: 11 million blocks, 5.7 GB of block values (byte offsets
+    beyond 2^31).  Blocked on the device; compact kernel (the plan's choice) and row-wise kernel."""
+    import torch
+    d = gen.rmat(20, 16)
+    M, K, nnz = d["M"], d["K"], int(d["row_ptr"][-1])
+    N = 128
+    dev = smat.csr_to_bcsr_device(M, K, to_dev(torch, d["row_ptr"], cuda), to_dev(torch, d["col_idx"], cuda),
+                                  to_dev(torch, d["val"], cuda), nnz)
+    nnzb = dev.nnzb
+    assert nnzb * 512 > 2**32
+    host = dev.to_host()
+    A = {"M": M, "K": K, "b_row_ptr": host.row_ptr, "b_col_idx": host.col_idx, "b_val": host.val, "nnzb": nnzb}
+    mb = M // 16
+    heaviest = int(np.argmax(np.diff(host.row_ptr)))
+    rows = sample_rows(mb, 12, extra=(heaviest, mb - 1, mb - 2))  # the last rows read the highest offsets
+    B = gen.dense_b(K, N, seed=0xB0000003, dist="uniform")
+    B2 = (B.view(np.float16) * np.float16(2)).view(np.uint16)
+
+    class Ptr:  # the arrays the device blocking returned, for smat.spmm / Plan.attach_values
+        def __init__(self, p):
+            self.p = p
+
+        def data_ptr(self):
+            return self.p
+    vals, rp, ci = Ptr(dev.val), Ptr(dev.row_ptr), Ptr(dev.col_idx)
+    Bd, B2d = to_dev(torch, B, cuda), to_dev(torch, B2, cuda)
+    plan = smat.Plan(host.row_ptr, M, K, nnzb, N, col_idx_host=host.col_idx, kernel=0)
+    plan.attach_values(vals, rp, ci)
+    assert plan.info()["kernel"] == 5
+    C = torch.full((M, N), 0x7E00, dtype=torch.int16, device=cuda)
+    smat.spmm(vals, rp, ci, Bd, C, M, N, K, nnzb, plan=plan)
+    torch.cuda.synchronize()
+    check_sampled(oracle, A, B, N, C.cpu().numpy().view(np.uint16), rows)
+    # linearity in B: A (2 B) = 2 (A B) bit for bit, fp16 output included (no result near the fp16 limits)
+    C2 = torch.full((M, N), 0x7E00, dtype=torch.int16, device=cuda)
+    smat.spmm(vals, rp, ci, B2d, C2, M, N, K, nnzb, plan=plan)
+    torch.cuda.synchronize()
+    c, c2 = C.view(torch.float16), C2.view(torch.float16)
+    assert bool(torch.isfinite(c2).all()) and float(c.abs().max()) < 30000
+    tiny = c.abs() < 2.0**-13  # twice a subnormal result may round differently
+    assert bool(((c * 2 == c2) | tiny).all())
+    plan.close()
+    # row-wise kernel through the drop-in entry point (no plan): same sampled rows
+    C.fill_(0x7E00)
+    smat.spmm(vals, rp, ci, Bd, C, M, N, K, nnzb, drop_in=True)
+    torch.cuda.synchronize()
+    check_sampled(oracle, A, B, N, C.cpu().numpy().view(np.uint16), rows)
+    dev.close()
+
+
+def test_config2_reordered_full_size(smat, cuda, oracle):
+    """Config 2 (16384 x 16384, 0.1 %, N = 256) after both reorder passes: whole result against the oracle,
+    and equal to the product of the unpermuted matrix with rows and B permuted accordingly."""
+    d = gen.erdos_renyi(16384, 0.001)
+    pr, pc, sr, sc = smat.reorder_csr(d["M"], d["K"], d["row_ptr"], d["col_idx"], 16, 16, 0.5, True)
+    rp, ci, v = smat.permute_csr(d["M"], d["K"], d["row_ptr"], d["col_idx"], d["val"], pr, pc)
+    A = bcsr_of(smat, {"M": d["M"], "K": d["K"], "row_ptr": rp, "col_idx": ci, "val": v})
+    assert A["nnzb"] == sc[2] < bcsr_of(smat, d)["nnzb"]
+    N = 256
+    B = gen.dense_b(A["K"], N, seed=0xB0000002, dist="normal")
+    C, info = gpu_spmm_compact(smat, cuda, A, B, N, kernel=0)
+    assert info["kernel"] == 5
+    assert oracle.compare(C, oracle_ref(oracle, A, B, N))[0] <= TOL_F16
+    # P_r A P_c times B  ==  P_r (A times (P_c B)): row i of the reordered product is row pr[i] of the
+    # product of the original matrix with the rows of B moved back (same tolerance, other summation order)
+    Bm = B.reshape(N, A["K"])                      # column-major: [n][k]
+    B_back = np.empty_like(Bm)
+    B_back[:, pc] = Bm                             # row pc[j] of the original B' is row j of B
+    ref = oracle.spmm_csr(d["M"], N, d["K"], d["row_ptr"], d["col_idx"], d["val"], B_back.ravel())
+    assert oracle.compare(C, ref[pr])[0] <= TOL_F16
+
+
+@pytest.mark.parametrize("reordered", [False, True])
+def test_config5_stencil_64_full_size(smat, cuda, oracle, reordered):
+    """27-point stencil on a 64^3 grid (262,144 rows), N = 64: sampled block rows against the oracle."""
+    d = gen.stencil27(64)
+    if reordered:
+        pr, pc, sr, sc = smat.reorder_csr(d["M"], d["K"], d["row_ptr"], d["col_idx"], 16, 16, 0.5, True)
+        rp, ci, v = smat.permute_csr(d["M"], d["K"], d["row_ptr"], d["col_idx"], d["val"], pr, pc)
+        d = {"M": d["M"], "K": d["K"], "row_ptr": rp, "col_idx": ci, "val": v}
+    A = bcsr_of(smat, d)
+    N = 64
+    B = gen.dense_b(A["K"], N, seed=0xB0000005, dist="uniform")
+    C, info = gpu_spmm_compact(smat, cuda, A, B, N, kernel=0)
+    mb = A["M"] // 16
+    check_sampled(oracle, A, B, N, C, sample_rows(mb, 40, extra=(1, mb - 2)))
+    # the row-wise kernel on the same operands: close to it everywhere (other summation order)
+    C1, _ = gpu_spmm_compact(smat, cuda, A, B, N, kernel=1)
+    a, b = C.view(np.float16).astype(np.float32), C1.view(np.float16).astype(np.float32)
+    assert np.abs(a - b).max() <= 2e-3 * np.abs(b).max()

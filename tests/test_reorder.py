@@ -93,6 +93,66 @@ def test_live_against_reference_program_stencil_32k_rows(smat, tmp_path):
     assert np.array_equal(g, want)
 
 
+TWO_PASS = sorted(glob.glob(os.path.join(HERE, "golden", "reorder_two_pass", "*.npz")))
+
+
+def check_two_pass(smat, rows, cols, row_ptr, col_idx, cb, rb, tau, want):
+    """smat_reorder_csr (row pass, then the same pass on the transpose of the row-permuted pattern) against
+    the two runs of the reference program, src/reorder.py:107-182: per pass the reordered edge list, the
+    counters, and that the permutation sorts the rows by the GROUPING line."""
+    M, K = rows + 5, cols + 3  # trailing empty rows / columns: not in an edge list, they keep their place
+    rp = np.concatenate([row_ptr, np.full(5, row_ptr[-1])]).astype(np.int32)
+    pr, pc, sr, sc = smat.reorder_csr(M, K, rp, col_idx, cb, rb, tau, do_cols=True)
+    assert np.array_equal(np.sort(pr), np.arange(M)) and np.array_equal(np.sort(pc), np.arange(K))
+    assert np.array_equal(pr[rows:], np.arange(rows, M)) and np.array_equal(pc[cols:], np.arange(cols, K))
+    pr, pc = pr[:rows], pc[:cols]
+    # row pass
+    nr, nc = reordered_edges(rows, row_ptr, col_idx, pr)
+    assert np.array_equal(nr, want["row_pass_el"][:, 0]) and np.array_equal(nc, want["row_pass_el"][:, 1])
+    assert np.array_equal(sr, want["stats_rows"])
+    assert np.all(np.diff(want["grouping_rows"][pr]) >= 0)
+    # column pass: the rows of the transpose are the columns; its edge list after the pass is
+    # (new column, new row) sorted by new column, the new rows of a column ascending
+    inv_c = np.empty(cols, np.int64)
+    inv_c[pc] = np.arange(cols)
+    t_rows, t_cols = inv_c[nc], nr
+    order = np.lexsort((t_cols, t_rows))
+    assert np.array_equal(t_rows[order], want["col_pass_el"][:, 0]) and np.array_equal(t_cols[order], want["col_pass_el"][:, 1])
+    assert np.array_equal(sc, want["stats_cols"])
+    assert want["grouping_cols"].size == cols and np.all(np.diff(want["grouping_cols"][pc]) >= 0)
+
+
+def test_two_pass_fixtures_exist():
+    assert len(TWO_PASS) >= 5
+
+
+@pytest.mark.parametrize("path", TWO_PASS, ids=[os.path.basename(p)[:-4] for p in TWO_PASS])
+def test_column_pass_matches_reference_on_the_transposed_row_permuted_edge_list(smat, path):
+    d = np.load(path)
+    cb, rb, tau = d["params"]
+    check_two_pass(smat, int(d["rows"]), int(d["cols"]), d["row_ptr"], d["col_idx"], int(cb), int(rb), float(np.float32(tau)), d)
+
+
+@pytest.mark.skipif(ref_binary("Matrix_Blocking") is None, reason="oracle/_ref/Matrix_Blocking not built")
+@pytest.mark.parametrize("seed", range(4))
+def test_two_pass_live_against_reference_program(smat, tmp_path, seed):
+    import sys
+    sys.path.insert(0, os.path.join(HERE, "golden"))
+    import make_reorder_golden as mk
+    rng = np.random.default_rng(100 + seed)
+    rows, cols = int(rng.integers(100, 900)), int(rng.integers(100, 1200))
+    nnz = int(rows * rng.uniform(2, 10))
+    key = np.unique(np.concatenate([rng.integers(0, rows, nnz) * cols + rng.integers(0, cols, nnz),
+                                    [(rows - 1) * cols + cols - 1]]))
+    r, c = key // cols, key % cols
+    cb, rb, tau = [(16, 16, 0.5), (8, 16, 0.5), (16, 16, 0.3), (4, 6, 0.6)][seed]
+    (g1, el1, st1), (g2, el2, st2) = mk.run_two_pass(r, c, cb, rb, tau, str(tmp_path))
+    row_ptr = np.zeros(rows + 1, dtype=np.int64)
+    np.add.at(row_ptr, r + 1, 1)
+    want = {"row_pass_el": el1, "col_pass_el": el2, "stats_rows": st1, "stats_cols": st2, "grouping_rows": g1, "grouping_cols": g2}
+    check_two_pass(smat, rows, cols, np.cumsum(row_ptr), c, cb, rb, float(np.float32(tau)), want)
+
+
 def test_two_pass_flow_and_permute(smat):
     d = gen.stencil27(10)  # 1000 rows -> padded to 1008
     M = K = 1008
