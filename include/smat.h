@@ -68,10 +68,13 @@ int smat_spmm_bcsr_f16(const uint16_t *vals, const int32_t *row_ptr, const int32
 #define SMAT_KERNEL_AUTO 0
 #define SMAT_KERNEL_ROWWISE 1 /* one wavefront per (block-row chunk, N panel), operands straight from L2;
                                * the plan decides whether B is first repacked slab-major into scratch   */
-#define SMAT_KERNEL_SWEEP 2   /* workgroup sweeps K for a group of 32 block rows x 128 columns, B panel staged
-                               * in LDS; needs a plan made with col_idx_host, fewer than 2^23 blocks and a B
-                               * smaller than 4 GiB.  SMAT_KERNEL_AUTO takes it when at least 5% of the blocks
-                               * exist and (M/512) x (N/128) workgroups fill the 256 CUs                     */
+#define SMAT_KERNEL_SWEEP 2   /* workgroup sweeps K for a group of 64 block rows x 64 columns, B staged in LDS
+                               * in chunks of 16 block columns; needs a plan made with col_idx_host, between 2
+                               * and 2^23 - 1 blocks and K below 2^28.  SMAT_KERNEL_AUTO takes it when at least
+                               * 5% of the blocks exist and (M/1024) x (N/64) workgroups fill the 256 CUs.
+                               * It works from the plan's op list, NOT from the row_ptr / col_idx passed at
+                               * launch: the plan must have been made from the same block pattern
+                               * (smat_plan_check verifies that on request)                                 */
 #define SMAT_KERNEL_ROWWISE_DIRECT 3 /* row-wise, B always read in place (plan or launch option)          */
 #define SMAT_KERNEL_COMPACT 5  /* only the nonzero columns of the blocks are multiplied (needs
                                * smat_plan_attach_values); for blocks with few nonzero columns */
@@ -90,6 +93,15 @@ typedef struct smat_spmm_opts {
  * BCSR build (SparseMatrix ctor, matrix.h:173): made once per matrix, outside
  * the timed loop (tester.h:342-358), reused by every launch. */
 typedef struct smat_plan smat_plan;
+/* Contract of a plan:
+ *  - One launch in flight at a time.  Every launch with a plan writes plan-owned scratch (the repacked or
+ *    transposed copy of B, the partial sums of split block rows): two launches of one plan that overlap
+ *    (different streams, or one stream per thread) race and corrupt C without an error.  Launches on one
+ *    stream are ordered and safe; for concurrent launches make one plan per stream.
+ *  - A plan belongs to one block pattern.  The launch checks M, K and nnzb only; the sweep kernel takes the
+ *    pattern from the plan, the compact kernel the pattern and the values (as attached).  A plan made from
+ *    another matrix of the same size, or values changed without attaching them again, give a wrong C with
+ *    SMAT_OK.  smat_plan_check compares the fingerprint of the host arrays the plan was made from. */
 
 /* row_ptr_host: the HOST copy of the BCSR row pointer (M/16+1 entries).
  * col_idx_host: HOST copy of the BCSR column index (may be NULL unless
@@ -104,11 +116,17 @@ int smat_plan_create(smat_plan **plan, const int32_t *row_ptr_host, const int32_
  * SMAT_KERNEL_COMPACT multiplies only those and touches only the rows of B under them; with
  * SMAT_KERNEL_AUTO the plan switches to that kernel when fewer than 60% of the block columns
  * are nonzero.  The compact kernel works from the copy: attach again after the values change.
- * Synchronous.  No counterpart in the reference, which multiplies every block as a dense
+ * The new list is built before the old one is dropped; if the call fails the plan has no list and
+ * SMAT_KERNEL_AUTO goes back to the sweep or row-wise kernel.  Synchronous.  No counterpart in the reference, which multiplies every block as a dense
  * 16x16 (mmaCBT.cu:44-66). */
 int smat_plan_attach_values(smat_plan *plan, const uint16_t *vals, const int32_t *row_ptr,
                             const int32_t *col_idx, const int32_t *row_ptr_host);
 int smat_plan_destroy(smat_plan *plan);
+/* Opt-in check that `plan` was made from this block pattern: M, K, nnzb and a 64-bit FNV-1a hash of
+ * row_ptr_host (and of col_idx_host if the plan was made with one; then it must be passed).  One pass over
+ * the host arrays; SMAT_ERR_INVALID when they differ.  No counterpart in the reference. */
+int smat_plan_check(const smat_plan *plan, const int32_t *row_ptr_host, const int32_t *col_idx_host,
+                    size_t M, size_t K, size_t nnzb);
 /* Fills info[0..9]: kernel id, row-wise work items, split block rows, chunk size,
  * workspace bytes, panel width, sweep MFMA ops, sweep (row group, K chunk) records,
  * bytes of the scratch copy of B (0 = B is read in place), nonzero block columns listed by

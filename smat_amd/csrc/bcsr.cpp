@@ -24,7 +24,7 @@
 
 using namespace smat;
 
-extern "C" int smat_csr_to_bcsr(size_t M, size_t K, const int32_t *row_ptr, const int32_t *col_idx,
+static int smat_csr_to_bcsr_impl(size_t M, size_t K, const int32_t *row_ptr, const int32_t *col_idx,
                                  const uint16_t *val, int64_t *counts, int32_t **b_row_ptr,
                                  int32_t **b_col_idx, uint16_t **b_val, int32_t **block_info,
                                  int32_t **rel_map)
@@ -126,4 +126,12 @@ extern "C" int smat_csr_to_bcsr(size_t M, size_t K, const int32_t *row_ptr, cons
     }
     *b_row_ptr = orp; *b_col_idx = oci; *b_val = ov;
     return SMAT_OK;
+}
+
+extern "C" int smat_csr_to_bcsr(size_t M, size_t K, const int32_t *row_ptr, const int32_t *col_idx,
+                                 const uint16_t *val, int64_t *counts, int32_t **b_row_ptr,
+                                 int32_t **b_col_idx, uint16_t **b_val, int32_t **block_info,
+                                 int32_t **rel_map)
+{
+    return smat::guarded("smat_csr_to_bcsr", [&] { return smat_csr_to_bcsr_impl(M, K, row_ptr, col_idx, val, counts, b_row_ptr, b_col_idx, b_val, block_info, rel_map); });
 }

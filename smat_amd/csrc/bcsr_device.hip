@@ -153,7 +153,7 @@ struct Scratch {
 
 } // namespace
 
-extern "C" int smat_csr_to_bcsr_device(size_t M, size_t K, const int32_t *row_ptr, const int32_t *col_idx,
+static int smat_csr_to_bcsr_device_impl(size_t M, size_t K, const int32_t *row_ptr, const int32_t *col_idx,
                                         const uint16_t *val, size_t nnz, int64_t *counts,
                                         int32_t **b_row_ptr, int32_t **b_col_idx, uint16_t **b_val)
 {
@@ -260,4 +260,11 @@ extern "C" int smat_csr_to_bcsr_device(size_t M, size_t K, const int32_t *row_pt
     *b_row_ptr = orp; *b_col_idx = oci; *b_val = ov;
     return SMAT_OK;
 #undef SMAT_TRY
+}
+
+extern "C" int smat_csr_to_bcsr_device(size_t M, size_t K, const int32_t *row_ptr, const int32_t *col_idx,
+                                        const uint16_t *val, size_t nnz, int64_t *counts,
+                                        int32_t **b_row_ptr, int32_t **b_col_idx, uint16_t **b_val)
+{
+    return smat::guarded("smat_csr_to_bcsr_device", [&] { return smat_csr_to_bcsr_device_impl(M, K, row_ptr, col_idx, val, nnz, counts, b_row_ptr, b_col_idx, b_val); });
 }

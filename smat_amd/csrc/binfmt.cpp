@@ -75,7 +75,7 @@ int write_file(const char *path, uint32_t kind, size_t M, size_t K, size_t n, co
 
 } // namespace
 
-extern "C" int smat_bin_write_csr(const char *path, size_t M, size_t K, const int32_t *row_ptr,
+static int smat_bin_write_csr_impl(const char *path, size_t M, size_t K, const int32_t *row_ptr,
                                    const int32_t *col_idx, const uint16_t *val, const int64_t *perm_rows,
                                    const int64_t *perm_cols)
 {
@@ -90,7 +90,14 @@ extern "C" int smat_bin_write_csr(const char *path, size_t M, size_t K, const in
     return write_file(path, 1, M, K, nnz, sec, n_sec, flags);
 }
 
-extern "C" int smat_bin_write_bcsr(const char *path, size_t M, size_t K, size_t nnzb, const int32_t *b_row_ptr,
+extern "C" int smat_bin_write_csr(const char *path, size_t M, size_t K, const int32_t *row_ptr,
+                                   const int32_t *col_idx, const uint16_t *val, const int64_t *perm_rows,
+                                   const int64_t *perm_cols)
+{
+    return smat::guarded("smat_bin_write_csr", [&] { return smat_bin_write_csr_impl(path, M, K, row_ptr, col_idx, val, perm_rows, perm_cols); });
+}
+
+static int smat_bin_write_bcsr_impl(const char *path, size_t M, size_t K, size_t nnzb, const int32_t *b_row_ptr,
                                     const int32_t *b_col_idx, const uint16_t *b_val, const int64_t *perm_rows,
                                     const int64_t *perm_cols)
 {
@@ -106,7 +113,14 @@ extern "C" int smat_bin_write_bcsr(const char *path, size_t M, size_t K, size_t 
     return write_file(path, 2, M, K, nnzb, sec, n_sec, flags);
 }
 
-extern "C" int smat_bin_read(const char *path, int *kind, size_t *M, size_t *K, size_t *n, int32_t **row_ptr,
+extern "C" int smat_bin_write_bcsr(const char *path, size_t M, size_t K, size_t nnzb, const int32_t *b_row_ptr,
+                                    const int32_t *b_col_idx, const uint16_t *b_val, const int64_t *perm_rows,
+                                    const int64_t *perm_cols)
+{
+    return smat::guarded("smat_bin_write_bcsr", [&] { return smat_bin_write_bcsr_impl(path, M, K, nnzb, b_row_ptr, b_col_idx, b_val, perm_rows, perm_cols); });
+}
+
+static int smat_bin_read_impl(const char *path, int *kind, size_t *M, size_t *K, size_t *n, int32_t **row_ptr,
                               int32_t **col_idx, uint16_t **val, int64_t **perm_rows, int64_t **perm_cols)
 {
     if (!path || !kind || !M || !K || !n || !row_ptr || !col_idx || !val)
@@ -121,7 +135,8 @@ extern "C" int smat_bin_read(const char *path, int *kind, size_t *M, size_t *K, 
         fclose(f);
         return set_error(SMAT_ERR_IO, "%s is not a SMATBIN1 file", path);
     }
-    if ((h.kind != 1 && h.kind != 2) || (h.flags & ~3u) || h.M > 0x7fffffffull * 16 || h.n > 0x7fffffffull ||
+    if ((h.kind != 1 && h.kind != 2) || (h.flags & ~3u) || h.M > 0x7fffffffull * 16 || h.K > 0x7fffffffull * 16 ||
+        h.n > 0x7fffffffull ||
         (h.kind == 2 && (h.M % 16 || h.K % 16))) {
         fclose(f);
         return set_error(SMAT_ERR_IO, "%s: inconsistent header", path);
@@ -147,6 +162,16 @@ extern "C" int smat_bin_read(const char *path, int *kind, size_t *M, size_t *K, 
     if (ok) {
         const int32_t *rp = static_cast<const int32_t *>(buf[0]);
         if (rp[0] != 0 || (uint64_t)rp[rows] != h.n) { ok = false; rc = set_error(SMAT_ERR_IO, "%s: row pointer does not match the entry count", path); }
+        for (size_t r = 0; ok && r < rows; r++)
+            if (rp[r + 1] < rp[r]) { ok = false; rc = set_error(SMAT_ERR_IO, "%s: row pointer decreases at row %zu", path, r); }
+        const int32_t *ci = static_cast<const int32_t *>(buf[1]);
+        const int32_t step = h.kind == 2 ? 16 : 1;
+        for (size_t e = 0; ok && e < h.n; e++)
+            if (ci[e] < 0 || (uint64_t)ci[e] >= h.K || ci[e] % step) {
+                ok = false;
+                rc = set_error(SMAT_ERR_IO, "%s: column index %d of entry %zu is not a %scolumn of K = %llu", path, ci[e], e,
+                               h.kind == 2 ? "block " : "", (unsigned long long)h.K);
+            }
     }
     if (!ok) {
         for (void *b : buf) free(b);
@@ -161,10 +186,16 @@ extern "C" int smat_bin_read(const char *path, int *kind, size_t *M, size_t *K, 
     return SMAT_OK;
 }
 
+extern "C" int smat_bin_read(const char *path, int *kind, size_t *M, size_t *K, size_t *n, int32_t **row_ptr,
+                              int32_t **col_idx, uint16_t **val, int64_t **perm_rows, int64_t **perm_cols)
+{
+    return smat::guarded("smat_bin_read", [&] { return smat_bin_read_impl(path, kind, M, K, n, row_ptr, col_idx, val, perm_rows, perm_cols); });
+}
+
 // CSR -> Matrix Market "coordinate real general", entries in storage order, 1-based; a value is
 // printed with enough digits to read back to the same fp16 (any fp16 is exact in 11 significant
 // decimal digits or fewer when printed from its double).
-extern "C" int smat_mtx_write(const char *path, size_t M, size_t K, const int32_t *row_ptr,
+static int smat_mtx_write_impl(const char *path, size_t M, size_t K, const int32_t *row_ptr,
                                const int32_t *col_idx, const uint16_t *val)
 {
     if (!path || !row_ptr) return set_error(SMAT_ERR_INVALID, "NULL argument");
@@ -177,4 +208,10 @@ extern "C" int smat_mtx_write(const char *path, size_t M, size_t K, const int32_
             fprintf(f, "%zu %d %.11g\n", r + 1, col_idx[j] + 1, (double)half_to_float(val[j]));
     if (fclose(f) != 0) return set_error(SMAT_ERR_IO, "short write to %s", path);
     return SMAT_OK;
+}
+
+extern "C" int smat_mtx_write(const char *path, size_t M, size_t K, const int32_t *row_ptr,
+                               const int32_t *col_idx, const uint16_t *val)
+{
+    return smat::guarded("smat_mtx_write", [&] { return smat_mtx_write_impl(path, M, K, row_ptr, col_idx, val); });
 }

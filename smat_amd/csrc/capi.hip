@@ -41,6 +41,8 @@ struct smat_plan {
     int n_rg = 0, n_records = 0, n_ops = 0;
     int32_t *d_rg_chunk_ptr = nullptr, *d_chunk_ids = nullptr, *d_op_ptr = nullptr, *d_row_map = nullptr;
     SweepOp *d_ops = nullptr;
+    uint64_t fingerprint = 0; // FNV-1a over row_ptr_host and, when given, col_idx_host
+    bool fingerprint_has_cols = false;
     // compacted-column kernel (present after smat_plan_attach_values)
     CompactPlan *compact = nullptr;
     uint16_t *d_bt = nullptr; // row-major copy of B, K * n_cap halves (compact kernel)
@@ -211,7 +213,27 @@ extern "C" int smat_spmm_bcsr_f16_static(const uint16_t *vals, const int32_t *ro
 
 // ---- plans -----------------------------------------------------------------
 
-extern "C" int smat_plan_create(smat_plan **out, const int32_t *row_ptr_host,
+static uint64_t fnv1a(uint64_t h, const void *data, size_t bytes)
+{
+    const unsigned char *p = static_cast<const unsigned char *>(data);
+    for (size_t i = 0; i < bytes; i++) h = (h ^ p[i]) * 0x100000001b3ull;
+    return h;
+}
+static uint64_t pattern_fingerprint(const int32_t *row_ptr_host, const int32_t *col_idx_host, size_t mb, size_t nnzb)
+{
+    uint64_t h = fnv1a(0xcbf29ce484222325ull, row_ptr_host, (mb + 1) * sizeof(int32_t));
+    if (col_idx_host) h = fnv1a(h, col_idx_host, nnzb * sizeof(int32_t));
+    return h;
+}
+
+namespace {
+struct PlanHolder { // frees a half-built plan on every way out but the good one
+    smat_plan *p;
+    ~PlanHolder() { if (p) smat_plan_destroy(p); }
+};
+} // namespace
+
+static int smat_plan_create_impl(smat_plan **out, const int32_t *row_ptr_host,
                                  const int32_t *col_idx_host, size_t M, size_t K, size_t nnzb,
                                  size_t n_hint, const smat_spmm_opts *opts)
 {
@@ -236,8 +258,11 @@ extern "C" int smat_plan_create(smat_plan **out, const int32_t *row_ptr_host,
 
     smat_plan *p = new (std::nothrow) smat_plan();
     if (!p) return set_error(SMAT_ERR_NOMEM, "out of host memory");
+    PlanHolder holder{p};
     p->M = M; p->K = K; p->nnzb = nnzb; p->n_cap = n_hint;
     p->kernel_requested = want;
+    p->fingerprint = pattern_fingerprint(row_ptr_host, col_idx_host, mb, nnzb);
+    p->fingerprint_has_cols = col_idx_host != nullptr;
 
     // A block row is split when it is much longer than the average: chunks of
     // `chunk` blocks (even, so block pairs stay aligned with the MFMA K = 32).
@@ -306,10 +331,8 @@ extern "C" int smat_plan_create(smat_plan **out, const int32_t *row_ptr_host,
         (double)nnzb >= 0.05 * (double)mb * (double)kb)
         sweep = true;
     if (sweep && (nnzb >= (size_t)1 << 23 || nnzb < 2)) { // blocks are addressed in pairs, with 32-bit byte offsets
-        if (want == SMAT_KERNEL_SWEEP) {
-            smat_plan_destroy(p);
+        if (want == SMAT_KERNEL_SWEEP)
             return set_error(SMAT_ERR_UNSUPPORTED, "SMAT_KERNEL_SWEEP takes between 2 and 2^23 - 1 nonzero blocks");
-        }
         sweep = false;
     }
     if (e == hipSuccess && sweep) {
@@ -335,23 +358,34 @@ extern "C" int smat_plan_create(smat_plan **out, const int32_t *row_ptr_host,
             p->d_bpack = nullptr;
         }
     }
-    if (e != hipSuccess) {
-        smat_plan_destroy(p);
-        return set_error(SMAT_ERR_HIP, "plan allocation failed: %s", hipGetErrorString(e));
-    }
+    if (e != hipSuccess) return set_error(SMAT_ERR_HIP, "plan allocation failed: %s", hipGetErrorString(e));
+    holder.p = nullptr;
     *out = p;
     return SMAT_OK;
 }
 
-extern "C" int smat_plan_attach_values(smat_plan *p, const uint16_t *vals, const int32_t *row_ptr,
+extern "C" int smat_plan_create(smat_plan **out, const int32_t *row_ptr_host,
+                                 const int32_t *col_idx_host, size_t M, size_t K, size_t nnzb,
+                                 size_t n_hint, const smat_spmm_opts *opts)
+{
+    return smat::guarded("smat_plan_create", [&] { return smat_plan_create_impl(out, row_ptr_host, col_idx_host, M, K, nnzb, n_hint, opts); });
+}
+
+static int smat_plan_attach_values_impl(smat_plan *p, const uint16_t *vals, const int32_t *row_ptr,
                                         const int32_t *col_idx, const int32_t *row_ptr_host)
 {
     if (!p || !row_ptr || !row_ptr_host) return set_error(SMAT_ERR_INVALID, "plan, row_ptr and row_ptr_host must not be NULL");
     if (p->nnzb && (!vals || !col_idx)) return set_error(SMAT_ERR_INVALID, "vals and col_idx must not be NULL");
-    if (p->compact) { compact_destroy(p->compact); p->compact = nullptr; }
+    // The new list is built before the old one goes.  Whatever happens below, the old list describes values
+    // that have changed, so it is dropped, and a plan left without a list goes back to a dense kernel.
     CompactPlan *c = nullptr;
     hipError_t e = compact_build(vals, row_ptr, col_idx, row_ptr_host, p->M / 16, p->nnzb, p->n_cap, &c);
-    if (e != hipSuccess) return set_error(SMAT_ERR_HIP, "attaching values failed: %s", hipGetErrorString(e));
+    if (p->compact) { compact_destroy(p->compact); p->compact = nullptr; }
+    const int dense_kernel = p->d_ops ? SMAT_KERNEL_SWEEP : SMAT_KERNEL_ROWWISE;
+    if (e != hipSuccess) {
+        if (p->kernel == SMAT_KERNEL_COMPACT) p->kernel = dense_kernel;
+        return set_error(SMAT_ERR_HIP, "attaching values failed: %s", hipGetErrorString(e));
+    }
     // The dense kernels gather 16 rows of B per block, this one a row per nonzero column.  Measured:
     // 7 nonzero columns per block (27-point stencil) 53 us against 86 us row-wise; 16 per block
     // (dense blocks, N = 4096) 326 us against 180 us.  The plan's choice below 60% of the columns
@@ -360,12 +394,13 @@ extern "C" int smat_plan_attach_values(smat_plan *p, const uint16_t *vals, const
                       (p->kernel_requested == SMAT_KERNEL_AUTO && (double)c->n_cols < 0.6 * 16.0 * (double)p->nnzb);
     if (!take) { // nothing will use the list: the plan keeps (or goes back to) a dense kernel
         compact_destroy(c);
-        if (p->kernel == SMAT_KERNEL_COMPACT) p->kernel = p->d_ops ? SMAT_KERNEL_SWEEP : SMAT_KERNEL_ROWWISE;
+        if (p->kernel == SMAT_KERNEL_COMPACT) p->kernel = dense_kernel;
         return SMAT_OK;
     }
     if (!p->d_bt) e = hipMalloc(&p->d_bt, p->K * p->n_cap * sizeof(uint16_t));
     if (e != hipSuccess) {
         compact_destroy(c);
+        if (p->kernel == SMAT_KERNEL_COMPACT) p->kernel = dense_kernel;
         return set_error(SMAT_ERR_HIP, "attaching values failed: %s", hipGetErrorString(e));
     }
     p->compact = c;
@@ -375,6 +410,12 @@ extern "C" int smat_plan_attach_values(smat_plan *p, const uint16_t *vals, const
         p->d_bpack = nullptr;
     }
     return SMAT_OK;
+}
+
+extern "C" int smat_plan_attach_values(smat_plan *p, const uint16_t *vals, const int32_t *row_ptr,
+                                        const int32_t *col_idx, const int32_t *row_ptr_host)
+{
+    return smat::guarded("smat_plan_attach_values", [&] { return smat_plan_attach_values_impl(p, vals, row_ptr, col_idx, row_ptr_host); });
 }
 
 extern "C" int smat_plan_destroy(smat_plan *p)
@@ -392,6 +433,20 @@ extern "C" int smat_plan_destroy(smat_plan *p)
     if (p->d_row_map) (void)hipFree(p->d_row_map);
     if (p->d_ops) (void)hipFree(p->d_ops);
     delete p;
+    return SMAT_OK;
+}
+
+extern "C" int smat_plan_check(const smat_plan *p, const int32_t *row_ptr_host, const int32_t *col_idx_host,
+                               size_t M, size_t K, size_t nnzb)
+{
+    if (!p || !row_ptr_host) return set_error(SMAT_ERR_INVALID, "plan and row_ptr_host must not be NULL");
+    if (p->M != M || p->K != K || p->nnzb != nnzb)
+        return set_error(SMAT_ERR_INVALID, "plan was built for another matrix (M/K/nnzb differ)");
+    if (p->fingerprint_has_cols && !col_idx_host)
+        return set_error(SMAT_ERR_INVALID, "the plan was built with col_idx_host: pass it to check the plan");
+    const uint64_t h = pattern_fingerprint(row_ptr_host, p->fingerprint_has_cols ? col_idx_host : nullptr, M / 16, nnzb);
+    if (h != p->fingerprint)
+        return set_error(SMAT_ERR_INVALID, "plan was built for another block pattern (row_ptr / col_idx differ)");
     return SMAT_OK;
 }
 

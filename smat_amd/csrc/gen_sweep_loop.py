@@ -127,6 +127,12 @@ def desc_scalar(slot, buf):
 
 def mfma_dispatch(J):
     w3 = ring(J, 3)
+    if "jump" in ABL:                                            # always block row 0, no jump
+        emit("s_nop 1")
+        for t in range(4):
+            acc = f"a[{4 * t}:{4 * t + 3}]"
+            emit(f"v_mfma_f32_16x16x32_f16 {acc}, {bset(J, t)}, {aslot(J)}, {acc}")
+        return
     emit(f"s_lshr_b32 s{S_T0}, {w3}, 23")                        # block row * 40
     emit("s_getpc_b64 vcc")
     label(f"Lpc_{J}")
@@ -242,14 +248,17 @@ def step(J):
     # LDS returns in order: per step one descriptor read, then four B reads.  What the step before the
     # previous one issued is needed now (B operands of this op, descriptor of op i + DQ - 1); the five reads
     # of the previous step may still be under way.
-    emit("s_waitcnt lgkmcnt(5)")
-    desc_scalar(J + DQ - 1, J)                                   # read two steps ago into buffer J % 2
-    desc_read(J)                                                 # op i + DQ + 1
+    if "lgkm" not in ABL:
+        emit("s_waitcnt lgkmcnt(5)")
+    if "desc" not in ABL:
+        desc_scalar(J + DQ - 1, J)                               # read two steps ago into buffer J % 2
+        desc_read(J)                                             # op i + DQ + 1
     b_reads(J + PB, J + PB)
     a_load(J + AHEAD, J + AHEAD, f"s{J}")
     emit(f"s_cmp_lt_u32 s{S_AGE}, {AHEAD}")
     emit(f"s_cbranch_scc1 Lvmslow_{J}_%=")
-    emit(f"s_waitcnt vmcnt({AHEAD})")
+    if "vm" not in ABL:
+        emit(f"s_waitcnt vmcnt({AHEAD})")
     label(f"Lvmdone_{J}")
     emit(f"s_add_u32 s{S_AGE}, s{S_AGE}, 1")
     mfma_dispatch(J)

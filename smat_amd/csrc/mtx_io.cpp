@@ -61,7 +61,7 @@ std::string lower(std::string s)
 
 extern "C" void smat_host_free(void *p) { free(p); }
 
-extern "C" int smat_mtx_read(const char *path, size_t *M, size_t *K, size_t *nnz_out,
+static int smat_mtx_read_impl(const char *path, size_t *M, size_t *K, size_t *nnz_out,
                               int *is_symmetric, int32_t **row_ptr, int32_t **col_idx,
                               uint16_t **val, int *ref_code)
 {
@@ -114,6 +114,12 @@ extern "C" int smat_mtx_read(const char *path, size_t *M, size_t *K, size_t *nnz
         return set_error(SMAT_ERR_IO, "%s: bad size line", path);
     }
     const long m = (m0 + 15) / 16 * 16, n = (n0 + 15) / 16 * 16;
+    // an entry takes at least "1 1\n": a count the rest of the file cannot hold is a garbled size line,
+    // and the CSR indices are int32
+    if ((size_t)nz > (size_t)(c.end - c.p) / 4 + 1 || m0 > 0x7ffffff0L || n0 > 0x7ffffff0L || nz > 0x3fffffffL) {
+        if (ref_code) *ref_code = -4;
+        return set_error(SMAT_ERR_IO, "%s: size line '%ld %ld %ld' does not fit the file or the int32 index range", path, m0, n0, nz);
+    }
 
     std::vector<int32_t> ri((size_t)nz), ci((size_t)nz);
     std::vector<uint16_t> vv((size_t)nz);
@@ -163,4 +169,11 @@ extern "C" int smat_mtx_read(const char *path, size_t *M, size_t *K, size_t *nnz
     if (is_symmetric) *is_symmetric = sym ? 1 : 0;
     *row_ptr = rp; *col_idx = cj; *val = cv;
     return SMAT_OK;
+}
+
+extern "C" int smat_mtx_read(const char *path, size_t *M, size_t *K, size_t *nnz_out,
+                              int *is_symmetric, int32_t **row_ptr, int32_t **col_idx,
+                              uint16_t **val, int *ref_code)
+{
+    return smat::guarded("smat_mtx_read", [&] { return smat_mtx_read_impl(path, M, K, nnz_out, is_symmetric, row_ptr, col_idx, val, ref_code); });
 }

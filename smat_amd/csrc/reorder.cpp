@@ -509,7 +509,7 @@ int reorder_rows_impl(int64_t rows, int64_t cols, const int64_t *row_ptr, const 
 
 using namespace smat;
 
-extern "C" int smat_reorder_rows(int64_t rows, int64_t cols, const int64_t *row_ptr,
+static int smat_reorder_rows_impl(int64_t rows, int64_t cols, const int64_t *row_ptr,
                                   const int64_t *col_idx, int64_t col_block, int64_t row_block,
                                   float tau, int64_t *grouping, int64_t *perm, int64_t *stats)
 {
@@ -517,7 +517,14 @@ extern "C" int smat_reorder_rows(int64_t rows, int64_t cols, const int64_t *row_
                              stats);
 }
 
-extern "C" int smat_reorder_csr(size_t M, size_t K, const int32_t *row_ptr, const int32_t *col_idx,
+extern "C" int smat_reorder_rows(int64_t rows, int64_t cols, const int64_t *row_ptr,
+                                  const int64_t *col_idx, int64_t col_block, int64_t row_block,
+                                  float tau, int64_t *grouping, int64_t *perm, int64_t *stats)
+{
+    return smat::guarded("smat_reorder_rows", [&] { return smat_reorder_rows_impl(rows, cols, row_ptr, col_idx, col_block, row_block, tau, grouping, perm, stats); });
+}
+
+static int smat_reorder_csr_impl(size_t M, size_t K, const int32_t *row_ptr, const int32_t *col_idx,
                                  int64_t col_block, int64_t row_block, float tau, int do_cols,
                                  int64_t *perm_rows, int64_t *perm_cols, int64_t *stats_rows,
                                  int64_t *stats_cols)
@@ -577,7 +584,15 @@ extern "C" int smat_reorder_csr(size_t M, size_t K, const int32_t *row_ptr, cons
     return SMAT_OK;
 }
 
-extern "C" int smat_permute_csr(size_t M, size_t K, const int32_t *row_ptr, const int32_t *col_idx,
+extern "C" int smat_reorder_csr(size_t M, size_t K, const int32_t *row_ptr, const int32_t *col_idx,
+                                 int64_t col_block, int64_t row_block, float tau, int do_cols,
+                                 int64_t *perm_rows, int64_t *perm_cols, int64_t *stats_rows,
+                                 int64_t *stats_cols)
+{
+    return smat::guarded("smat_reorder_csr", [&] { return smat_reorder_csr_impl(M, K, row_ptr, col_idx, col_block, row_block, tau, do_cols, perm_rows, perm_cols, stats_rows, stats_cols); });
+}
+
+static int smat_permute_csr_impl(size_t M, size_t K, const int32_t *row_ptr, const int32_t *col_idx,
                                  const uint16_t *val, const int64_t *perm_rows,
                                  const int64_t *perm_cols, int32_t **out_row_ptr,
                                  int32_t **out_col_idx, uint16_t **out_val)
@@ -631,4 +646,12 @@ extern "C" int smat_permute_csr(size_t M, size_t K, const int32_t *row_ptr, cons
     rp[M] = (int32_t)o;
     *out_row_ptr = rp; *out_col_idx = ci; *out_val = vv;
     return SMAT_OK;
+}
+
+extern "C" int smat_permute_csr(size_t M, size_t K, const int32_t *row_ptr, const int32_t *col_idx,
+                                 const uint16_t *val, const int64_t *perm_rows,
+                                 const int64_t *perm_cols, int32_t **out_row_ptr,
+                                 int32_t **out_col_idx, uint16_t **out_val)
+{
+    return smat::guarded("smat_permute_csr", [&] { return smat_permute_csr_impl(M, K, row_ptr, col_idx, val, perm_rows, perm_cols, out_row_ptr, out_col_idx, out_val); });
 }

@@ -6,6 +6,7 @@
 #include <cstring>
 
 #include "../../include/smat.h"
+#include "errors.h"
 
 namespace smat {
 
@@ -183,7 +184,7 @@ void build_sweep_plan(const int32_t *row_ptr, const int32_t *col_idx, size_t mb,
 // Test hook (not part of smat.h): builds the work list on the host and hands it out.  Arrays are
 // allocated with malloc; release each with smat_host_free.  row_map: n_rg * 64 block rows (-1 = none).  counts[0..5] = row groups, listed
 // chunks, ops (with fillers, without padding), pairs, singles, fillers.
-extern "C" int smat_internal_sweep_plan(const int32_t *row_ptr, const int32_t *col_idx, size_t M, size_t K,
+static int smat_internal_sweep_plan_impl(const int32_t *row_ptr, const int32_t *col_idx, size_t M, size_t K,
                                          int32_t **rg_chunk_ptr, int32_t **chunk_ids, int32_t **op_ptr,
                                          uint32_t **ops, int32_t **row_map, int64_t *counts)
 {
@@ -213,4 +214,11 @@ extern "C" int smat_internal_sweep_plan(const int32_t *row_ptr, const int32_t *c
     counts[4] = (int64_t)p.n_singles;
     counts[5] = (int64_t)p.n_fillers;
     return SMAT_OK;
+}
+
+extern "C" int smat_internal_sweep_plan(const int32_t *row_ptr, const int32_t *col_idx, size_t M, size_t K,
+                                         int32_t **rg_chunk_ptr, int32_t **chunk_ids, int32_t **op_ptr,
+                                         uint32_t **ops, int32_t **row_map, int64_t *counts)
+{
+    return smat::guarded("smat_internal_sweep_plan", [&] { return smat_internal_sweep_plan_impl(row_ptr, col_idx, M, K, rg_chunk_ptr, chunk_ids, op_ptr, ops, row_map, counts); });
 }

@@ -217,6 +217,12 @@ class Plan:
         check(lib.smat_plan_create(C.byref(self._h), _p(rp), _p(ci), M, K, nnzb, n_hint, C.byref(opts)))
         self._rp_host = rp
 
+    def check(self, row_ptr_host, col_idx_host, M, K, nnzb):
+        """Raises SmatError unless the plan was made from this block pattern (fingerprint of the host arrays)."""
+        rp = np.ascontiguousarray(row_ptr_host, dtype=np.int32)
+        ci = None if col_idx_host is None else np.ascontiguousarray(col_idx_host, dtype=np.int32)
+        check(lib.smat_plan_check(self._h, _p(rp), _p(ci), M, K, nnzb))
+
     def attach_values(self, vals_dev, row_ptr_dev, col_idx_dev):
         """Let the plan list the nonzero columns of the blocks (device tensors of the same matrix)."""
         ptr = lambda t: C.c_void_p(t.data_ptr()) if t is not None else None  # noqa: E731

@@ -107,3 +107,23 @@ def test_converter_cli(tmp_path):
     assert c["kind"] == 2 and np.array_equal(c["perm_rows"], pr) and np.array_equal(c["perm_cols"], pc)
     assert np.array_equal(c["row_ptr"], b.row_ptr) and np.array_equal(c["col_idx"], b.col_idx)
     assert np.array_equal(c["val"], b.val)
+
+
+def test_reader_validates_the_arrays_it_hands_on(tmp_path):
+    """Files with a good checksum whose arrays are not a matrix: out-of-range or unaligned column, decreasing
+    row pointer."""
+    rp = np.array([0, 2, 3] + [3] * 14, np.int32)
+    v = np.array([1, 2, 3], np.uint16)
+    smat_amd.bin_write_csr(tmp_path / "col.smat", 16, 16, rp, np.array([0, 16, 3], np.int32), v)
+    with pytest.raises(smat_amd.SmatError, match="column index 16"):
+        smat_amd.bin_read(tmp_path / "col.smat")
+    bad_rp = np.array([0, 3, 2] + [3] * 14, np.int32)
+    smat_amd.bin_write_csr(tmp_path / "rp.smat", 16, 16, bad_rp, np.array([0, 1, 3], np.int32), v)
+    with pytest.raises(smat_amd.SmatError, match="row pointer decreases"):
+        smat_amd.bin_read(tmp_path / "rp.smat")
+    A = gen.random_bcsr(2, 3, 1.0, seed=1)
+    ci = A["b_col_idx"].copy()
+    ci[1] = 8  # not a multiple of 16
+    smat_amd.bin_write_bcsr(tmp_path / "blk.smat", A["M"], A["K"], A["b_row_ptr"], ci, A["b_val"])
+    with pytest.raises(smat_amd.SmatError, match="block column"):
+        smat_amd.bin_read(tmp_path / "blk.smat")

@@ -476,3 +476,30 @@ def test_compact_kernel_power_law_rows(smat, cuda, oracle):
     C32, _ = gpu_spmm_compact(smat, cuda, A, B, N, kernel=0, c_f32=True)
     C32_2, _ = gpu_spmm_compact(smat, cuda, A, B2, N, kernel=0, c_f32=True)
     assert np.array_equal(C32 * np.float32(2), C32_2)
+
+
+def test_plan_check_tells_patterns_apart(smat, cuda):
+    """Two matrices of the same M, K and nnzb: the launch cannot tell them apart, smat_plan_check can."""
+    A = gen.random_bcsr(20, 24, 0.25, seed=41)
+    nnzb = A["nnzb"]
+    ci2 = A["b_col_idx"].copy()
+    ci2[0] = (ci2[0] + 16) % A["K"] if nnzb == 1 or (ci2[0] + 16) % A["K"] != ci2[1] else (ci2[0] + 32) % A["K"]
+    plan = smat.Plan(A["b_row_ptr"], A["M"], A["K"], nnzb, 64, col_idx_host=A["b_col_idx"])
+    plan.check(A["b_row_ptr"], A["b_col_idx"], A["M"], A["K"], nnzb)
+    with pytest.raises(smat.SmatError, match="another block pattern"):
+        plan.check(A["b_row_ptr"], ci2, A["M"], A["K"], nnzb)
+    with pytest.raises(smat.SmatError, match="pass it"):
+        plan.check(A["b_row_ptr"], None, A["M"], A["K"], nnzb)
+    with pytest.raises(smat.SmatError, match="M/K/nnzb"):
+        plan.check(A["b_row_ptr"], A["b_col_idx"], A["M"], A["K"] + 16, nnzb)
+    plan.close()
+    plan = smat.Plan(A["b_row_ptr"], A["M"], A["K"], nnzb, 64)  # made without column indices: row pointer only
+    plan.check(A["b_row_ptr"], None, A["M"], A["K"], nnzb)
+    plan.check(A["b_row_ptr"], ci2, A["M"], A["K"], nnzb)
+    rp2 = A["b_row_ptr"].copy()
+    i = int(np.argmax(np.diff(rp2) > 0))
+    rp2[i + 1] -= 1 if i + 1 < rp2.size - 1 else 0
+    if not np.array_equal(rp2, A["b_row_ptr"]):
+        with pytest.raises(smat.SmatError, match="another block pattern"):
+            plan.check(rp2, None, A["M"], A["K"], nnzb)
+    plan.close()

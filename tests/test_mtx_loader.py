@@ -60,3 +60,12 @@ def test_band_file_like_the_reference_generator(oracle, smat, tmp_path):
     assert a["M"] == 112 and a["nnz"] == n * (2 * b + 1) - b * (b + 1)
     for key in ("row_ptr", "col_idx", "val"):
         assert np.array_equal(a[key], o[key])
+
+
+def test_garbled_size_line_is_an_error_not_an_abort(smat, tmp_path):
+    """An entry count the file cannot hold (or one that would need terabytes) comes back as an I/O error."""
+    for sizes in ("4 4 4000000000000", "4 4 99", "99999999999 4 1"):
+        p = tmp_path / "bad.mtx"
+        p.write_text(f"%%MatrixMarket matrix coordinate real general\n{sizes}\n1 1 1.0\n")
+        with pytest.raises(smat.SmatError, match="size line"):
+            smat.mtx_read(p)
