@@ -340,7 +340,7 @@ static int smat_plan_create_impl(smat_plan **out, const int32_t *row_ptr_host,
         build_sweep_plan(row_ptr_host, col_idx_host, mb, kb, h);
         p->kernel = SMAT_KERNEL_SWEEP;
         p->n_rg = (int)h.rg_chunk_ptr.size() - 1;
-        p->n_records = (int)h.chunk_ids.size();
+        p->n_records = (int)h.chunk_ids.size() - SWEEP_CHUNK_PAD;
         p->n_ops = (int)(h.ops.size() - SWEEP_OP_PAD);
         auto upload = [&](void **dst, const void *src, size_t bytes) {
             if (e != hipSuccess) return;

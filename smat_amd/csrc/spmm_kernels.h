@@ -1,6 +1,8 @@
 // Internal interface between the C ABI (capi.hip) and the kernel launchers.
 #pragma once
 #include <hip/hip_runtime.h>
+
+#include "sweep_format.h"
 #include <stddef.h>
 #include <stdint.h>
 
@@ -40,37 +42,7 @@ struct SpmmArgs {
     uint16_t *b_packed; // device scratch of K * N halves, or nullptr: read the column-major B directly
 };
 
-// One op of the sweep kernel: two blocks of the same block row that are neighbours in the BCSR
-// arrays (blocks q and q + 1), multiplied by one K = 32 MFMA per 16 columns.  The two blocks lie in
-// the same K chunk or in two consecutive chunks of the row group's chunk list.
-//   w0 = byte offset of block q in vals (q * 512)
-//   w1 = LDS byte offset (inside the ring of stages) of the 16 rows of B under block q
-//   w2 = offset of the rows under block q + 1, minus w1 (signed)
-//   w3 = flags in bits 0-2 | (local block row 0..7) * 40 << 23  (40 = bytes of code per block row in the
-//        kernel's computed jump to the MFMAs of that row)
-// LDS offset of ring slot s = (position of the chunk in the row group's chunk list % SWEEP_STAGES) *
-// SWEEP_S + block column inside the chunk:  (s / 8) * 16384 + (s % 8) * 32.
-// SWEEP_OP_ZERO_HI: block q + 1 does not belong to the op (unpaired block): its half is multiplied
-// by zeros.  SWEEP_OP_ZERO_LO: the same for block q (an unpaired last block of the matrix is listed
-// as the second half of the pair before it).  Both: a filler that multiplies zeros only and exists
-// so that every wavefront has at least two ops in every chunk.  SWEEP_OP_BOUNDARY: first op of a
-// chunk other than the first.
-struct SweepOp {
-    uint32_t w0, w1, w2, w3;
-};
-constexpr uint32_t SWEEP_OP_ZERO_HI = 1u << 0;
-constexpr uint32_t SWEEP_OP_ZERO_LO = 1u << 1;
-constexpr uint32_t SWEEP_OP_BOUNDARY = 1u << 2;
-
-// Geometry of the sweep kernel (fixed at compile time).
-constexpr int SWEEP_TN = 4;     // n-tiles of 16 per workgroup panel -> 64 columns
-constexpr int SWEEP_RW = 8;     // block rows per wavefront
-constexpr int SWEEP_WAVES = 8;  // wavefronts per workgroup
-constexpr int SWEEP_G = SWEEP_RW * SWEEP_WAVES; // 64 block rows per workgroup
-constexpr int SWEEP_S = 16;     // block columns (slabs) per K chunk
-constexpr int SWEEP_STAGES = 4; // chunks resident in LDS
-constexpr int SWEEP_MIN_OPS = 2; // ops per wavefront and chunk the kernel relies on (its LDS read-ahead)
-constexpr int SWEEP_OP_PAD = 384; // descriptor slots after the last op that the kernel reads ahead into (never executes)
+// Stream format and geometry of the sweep kernel: sweep_format.h (shared with the host-side plan builder).
 
 struct SweepArgs {
     const uint16_t *vals;
@@ -79,9 +51,9 @@ struct SweepArgs {
     size_t M, N, K, nnzb;
     bool c_f32;
     const int32_t *rg_chunk_ptr; // device, n_rg + 1: range of the row group in chunk_ids
-    const int32_t *chunk_ids;    // device: the K chunks in which the row group has blocks, ascending
+    const int32_t *chunk_ids;    // device: the K chunks in which the row group has blocks, ascending (+ SWEEP_CHUNK_PAD entries)
     const int32_t *op_ptr;       // device, n_rg * SWEEP_WAVES + 1: range of (row group, wavefront) in ops
-    const SweepOp *ops;          // device, op streams, SWEEP_OP_PAD slots of padding at the end
+    const SweepOp *ops;          // device, op streams (sweep_format.h)
     const int32_t *row_map;      // device, n_rg * SWEEP_G: block row of (row group, wavefront, local row), -1 = none
     int n_rg;
 };

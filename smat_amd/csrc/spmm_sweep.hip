@@ -13,25 +13,24 @@
 //    about the same work in every chunk) x 64 columns, 128 fp32 accumulator registers, and runs a
 //    host-built stream of ops.  One op = two blocks of one block row = one K = 32 step of
 //    v_mfma_f32_16x16x32_f16 per 16 columns (4 MFMAs).  The two blocks may sit in the same chunk or
-//    in two consecutive chunks (the ring keeps the previous stage), so few blocks stay unpaired; an
-//    unpaired block multiplies zeros in the upper K half.
-//  * Pipeline.  The op stream of a wavefront is one flat loop over the whole K sweep, unrolled by
-//    six: the B operands of an op are read from LDS two ops ahead (three register sets), its A
-//    operand (two neighbouring 512-byte blocks, one load straight into MFMA layout) comes from global
-//    memory four ops ahead (ring of six), its descriptor (16 bytes, offsets ready to use) is read
-//    six ops ahead from a window of the op stream that is itself copied into LDS 64 ops at a time.
-//    LDS reads are ordinary loads (the compiler counts them); everything that goes through the
-//    vector memory path (A loads, copies) is issued from inline assembly with explicit s_waitcnt
-//    vmcnt, because only the kernel knows which copies an A load does not have to wait for: vector
-//    memory instructions complete in order, and the number of younger ones is known at every wait.
-//  * Accumulators live in a[0:127] and are touched by inline assembly only: the block row of an op
-//    is a run-time value, and the choice between register sets is a branch between MFMA groups.
-//  * Synchronisation.  One barrier per chunk.  Entering chunk c: the copies of chunk c+1 (issued one
-//    chunk earlier) have landed, barrier, then the copies of chunk c+2 are issued into the stage
-//    that held chunk c-2.  Reads may therefore run ahead into chunk c+1 across the barrier.  The
-//    plan gives every wavefront at least two ops per chunk (zero-valued filler ops where a
-//    wavefront has fewer), so an op two ahead is never further than the next chunk and every
-//    wavefront passes every barrier.
+//    in two consecutive chunks (the ring keeps the previous stage), so few blocks stay unpaired.
+//  * Interpreter.  The stream of a wavefront is threaded code (gen_sweep_loop.py, sweep_format.h): every 16-byte
+//    entry carries the offset of the code block that executes it, a block ends in a jump to the block of the
+//    next entry.  Blocks are specialised for the stream position modulo 8 (register sets), the block row
+//    (accumulators) and the s_waitcnt the op needs, so an op costs its 4 MFMAs, 4 LDS reads, one A load, the
+//    address arithmetic of the reads, two waits and the jump: 18 instructions.  Entries come in through scalar
+//    loads, two at a time, six positions ahead.
+//  * Pipeline.  The B operands of an op are read from LDS one position ahead (two register sets), its A
+//    operand (two neighbouring 512-byte blocks, one load straight into MFMA layout) comes from global memory
+//    five positions ahead (ring of eight).  Vector memory operations complete in order, so the number of
+//    younger ones at every wait is known when the plan is built: 5, or 9 when a marker issued its copies in
+//    between.  A half of an MFMA that must not contribute (unpaired block) reads a 16 KiB region of zeros.
+//  * Accumulators live in a[0:127] and are touched by inline assembly only.
+//  * Synchronisation.  One barrier per chunk, in the marker entry that starts the chunk.  Marker of chunk c:
+//    the wavefront's own copies of chunk c (issued two markers earlier) have landed, barrier, then the copies
+//    of chunk c+2 go into the stage that held chunk c-2.  The plan gives every wavefront at least four ops
+//    per chunk (filler ops that multiply zeros where it has fewer), so markers are at least five positions
+//    apart and every wavefront passes every barrier.
 //
 // Same operand semantics as the reference launcher (src/cuda_hgemm/src/mma/mmaCBT.cu:83-88).
 #include <hip/hip_runtime.h>
@@ -55,16 +54,9 @@ constexpr int THREADS = 64 * W;                       // 512
 constexpr int ROW_BYTES = 256;                        // 8 slabs x 16 k x 2 B per n
 constexpr int STAGE_BYTES = (S / 8) * NT * ROW_BYTES; // 32768
 constexpr int COPIES = STAGE_BYTES / 1024 / W;        // copy instructions per wavefront and chunk: 4
-constexpr int PB = 2;                                 // B operands are read PB ops ahead (PB + 1 register sets)
-constexpr int DA = 6;                                 // A operand ring (register sets)
-constexpr int AHEAD = 4;                              // A operands are loaded AHEAD ops ahead (< DA)
-constexpr int DQ = 6;                                 // op descriptors are read from LDS DQ ops ahead (ring of DQ scalar pairs)
-constexpr int UNROLL = 6;                             // multiple of PB + 1, DA and DQ
-constexpr int WIN_SLOTS = 4;                          // descriptor windows (64 ops, 1 KiB) per wavefront in LDS; three are in use
-constexpr int WINDOW_BYTES = W * WIN_SLOTS * 1024;    // 32 KiB: with the four stages all 160 KiB of LDS
-static_assert(TN == 4 && RW == 8 && W == 8 && S == 16 && NS == 4 && COPIES == 4, "geometry the code below assumes");
-static_assert(UNROLL % (PB + 1) == 0 && UNROLL % DA == 0 && UNROLL % DQ == 0 && AHEAD < DA && AHEAD < DQ && PB < DQ,
-              "register sets are addressed by the unroll position");
+constexpr int ZERO_BYTES = 16384;                     // the region of zeros behind the stages
+static_assert(TN == 4 && RW == 8 && W == 8 && S == 16 && NS == 4 && COPIES == SWEEP_COPIES && STAGE_BYTES == (int)SWEEP_STAGE_BYTES,
+              "geometry the code below assumes");
 
 __device__ __forceinline__ void zero_accumulators()
 {
@@ -125,7 +117,10 @@ __global__ __launch_bounds__(THREADS) void spmm_sweep_kernel(
     const int per_xcd = gridDim.x >> 3;
     const int tile = (blockIdx.x & 7) * per_xcd + (blockIdx.x >> 3);
     if (tile >= total) return;
-    constexpr int RGB = 4;
+#ifndef SWEEP_RGB
+#define SWEEP_RGB 4
+#endif
+    constexpr int RGB = SWEEP_RGB;
     const int n_blk = (n_rg + RGB - 1) / RGB;
     int gb = tile / (RGB * n_panels);
     gb = gb < n_blk - 1 ? gb : n_blk - 1;
@@ -156,7 +151,6 @@ __global__ __launch_bounds__(THREADS) void spmm_sweep_kernel(
 
     const int c_begin = rg_chunk_ptr[rg], n_chunks = rg_chunk_ptr[rg + 1] - c_begin;
     const int op_begin = op_ptr[rg * W + wave];
-    const int n_ops = op_ptr[rg * W + wave + 1] - op_begin;
 
     if (n_chunks > 0) { // uniform over the workgroup: every wavefront has the chunk list of its row group
         auto lds_copy = [&](uint32_t voff, const void *sbase, uint32_t dst) { // 64 lanes x 16 B -> LDS dst + lane * 16
@@ -172,43 +166,47 @@ __global__ __launch_bounds__(THREADS) void spmm_sweep_kernel(
         const uint32_t ls = (uint32_t)((lane & 15) ^ (q | ((wave & 3) << 2)));
         const uint32_t k_lane = (uint32_t)(wave >> 2) * 128u + ls * 8u;  // k inside the chunk
         const uint32_t col_bytes = (uint32_t)q * (uint32_t)K * 2u;       // the launcher checks K < 2^28
-        const uint32_t kmax = (uint32_t)K - 8u;
+        const uint32_t copy_off = col_bytes + k_lane * 2u;               // byte offset of this lane's 16 bytes for chunk id 0
+        const uint32_t copy_lim = col_bytes + ((uint32_t)K - 8u) * 2u;   // slabs past K are referenced by no op: the read stays inside the matrix
         const uint32_t dst_wave = lbase + (uint32_t)(wave * COPIES) * 1024u;
-        // the four copy instructions of a chunk: scalar base = first of their four columns of B, bit `it` of
-        // copy_mask = those columns exist (N % 8 == 0: all four or none)
+        // the four copy instructions of a chunk: scalar base = first of their four columns of B.  Columns past N
+        // (last panel, N % 8 == 0) are replaced by the last four: what lands in their rows is never stored, and
+        // every wavefront issues the same number of copies (the plan counts them).
         const int col0 = n0 + (wave & 3) * 16;
-        const uint16_t *sb0 = B + (long)(col0 + 0) * K, *sb1 = B + (long)(col0 + 4) * K;
-        const uint16_t *sb2 = B + (long)(col0 + 8) * K, *sb3 = B + (long)(col0 + 12) * K;
-        const uint32_t copy_mask = __builtin_amdgcn_readfirstlane(
-            (col0 < N ? 1u : 0u) | (col0 + 4 < N ? 2u : 0u) | (col0 + 8 < N ? 4u : 0u) | (col0 + 12 < N ? 8u : 0u));
+        auto col_base = [&](int c) { return B + (long)(c + 4 <= N ? c : N - 4) * K; };
+        const uint16_t *sb0 = col_base(col0), *sb1 = col_base(col0 + 4), *sb2 = col_base(col0 + 8), *sb3 = col_base(col0 + 12);
         const int32_t *chunk_ptr = chunk_ids + c_begin;
         auto issue_copies = [&](int cl) { // chunk cl of the row group's list into stage cl % NS
-            uint32_t k = (uint32_t)chunk_ptr[cl] * (uint32_t)(S * 16) + k_lane;
-            k = k < kmax ? k : kmax; // slabs past K are referenced by no op; keep the read inside the matrix
-            const uint32_t voff = col_bytes + k * 2u;
+            uint32_t voff = (uint32_t)chunk_ptr[cl] * (uint32_t)(S * 16 * 2) + copy_off;
+            voff = voff < copy_lim ? voff : copy_lim;
             const uint32_t dst0 = dst_wave + (uint32_t)(cl % NS) * STAGE_BYTES;
-            if (copy_mask & 1) lds_copy(voff, sb0, dst0);
-            if (copy_mask & 2) lds_copy(voff, sb1, dst0 + 1024u);
-            if (copy_mask & 4) lds_copy(voff, sb2, dst0 + 2048u);
-            if (copy_mask & 8) lds_copy(voff, sb3, dst0 + 3072u);
+            lds_copy(voff, sb0, dst0);
+            lds_copy(voff, sb1, dst0 + 1024u);
+            lds_copy(voff, sb2, dst0 + 2048u);
+            lds_copy(voff, sb3, dst0 + 3072u);
         };
-        // ---- op descriptors: windows of 64 ops (1 KiB, one copy instruction), four LDS slots per wavefront ----
-        const SweepOp *op_base = ops + op_begin; // the plan pads the array: reads past n_ops stay inside it
-        const uint32_t win_lds = lbase + (uint32_t)(NS * STAGE_BYTES) + (uint32_t)wave * (WIN_SLOTS * 1024u);
-        const uint32_t lane16 = (uint32_t)lane * 16u;
-        // ---- prologue: chunks 0 and 1 and the descriptors of the first 192 ops resident ----
+        // ---- entry: chunks 0, 1, 2 on their way, the region of zeros written ----
         issue_copies(0);
         if (n_chunks > 1) issue_copies(1);
-        for (int wdw = 0; wdw < 3; wdw++) lds_copy(lane16, op_base + (long)wdw * 64, win_lds + (uint32_t)wdw * 1024u);
-        asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
-        __syncthreads();
+        if (n_chunks > 2) issue_copies(2);
+        {
+            i32x4 *zero = reinterpret_cast<i32x4 *>(lds + NS * STAGE_BYTES);
+            zero[tid] = i32x4{0, 0, 0, 0};
+            zero[tid + THREADS] = i32x4{0, 0, 0, 0};
+            static_assert(ZERO_BYTES == 2 * THREADS * 16, "two 16-byte stores per lane fill the region of zeros");
+        }
+        asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
 
-        // ---- the main loop: see gen_sweep_loop.py ----
+        // ---- the interpreter: see gen_sweep_loop.py ----
         const uint32_t rd_addr = lbase + (uint32_t)(16 * (i16 >> 2) + (i16 & 3)) * ROW_BYTES; // LDS address of this lane's column in stage 0
         const uint32_t a_voff = (uint32_t)sel * 512u + a_lane_bytes; // lanes 32-63 take the second block of the pair
         const uint32_t sel01 = (uint32_t)sel;
-        const uint32_t n_ops_u = __builtin_amdgcn_readfirstlane((uint32_t)n_ops), n_chunks_u = __builtin_amdgcn_readfirstlane((uint32_t)n_chunks);
-        const uint32_t op_lo = (uint32_t)(uintptr_t)op_base, op_hi = (uint32_t)((uintptr_t)op_base >> 32);
+        const uint32_t n_chunks_u = __builtin_amdgcn_readfirstlane((uint32_t)n_chunks);
+        const SweepOp *op_base = ops + op_begin;
+        const uint32_t op_lo = __builtin_amdgcn_readfirstlane((uint32_t)(uintptr_t)op_base);
+        const uint32_t op_hi = __builtin_amdgcn_readfirstlane((uint32_t)((uintptr_t)op_base >> 32));
+        const uint32_t chunk_lo = __builtin_amdgcn_readfirstlane((uint32_t)(uintptr_t)chunk_ptr);
+        const uint32_t chunk_hi = __builtin_amdgcn_readfirstlane((uint32_t)((uintptr_t)chunk_ptr >> 32));
 #ifndef SWEEP_LOOP_INC
 #define SWEEP_LOOP_INC "spmm_sweep_loop.inc"
 #endif
@@ -246,7 +244,7 @@ __global__ __launch_bounds__(THREADS) void spmm_sweep_kernel(
 
 hipError_t launch_sweep(const SweepArgs &a, hipStream_t st)
 {
-    const int lds_bytes = NS * STAGE_BYTES + WINDOW_BYTES;
+    const int lds_bytes = NS * STAGE_BYTES + ZERO_BYTES;
     // dynamic LDS above 64 KiB has to be allowed once per kernel and device; the call is cheap and idempotent
     hipError_t e = a.c_f32
         ? hipFuncSetAttribute(reinterpret_cast<const void *>(&spmm_sweep_kernel<true>),

@@ -5,23 +5,18 @@
 #include <cstdlib>
 #include <cstring>
 
+#include <stdexcept>
+
 #include "../../include/smat.h"
 #include "errors.h"
+#include "sweep_format.h"
 
 namespace smat {
 
 namespace {
-// mirrors spmm_kernels.h (that header needs the HIP runtime; this file is compiled by g++)
-constexpr uint32_t OP_ZERO_HI = 1u << 0, OP_ZERO_LO = 1u << 1, OP_BOUNDARY = 1u << 2;
-constexpr int G = 64, RW = 8, WAVES = 8, S = 16, STAGES = 4, MIN_OPS = 2, OP_PAD = 384;
-constexpr uint32_t ROW_CODE = 40; // bytes of code per block row in the kernel's MFMA dispatch
-
-// LDS byte offset of the 16 rows of B under a block: chunk position in the row group's list, block column in the chunk
-uint32_t lds_offset(int32_t chunk_pos, int32_t slab)
-{
-    const uint32_t slot = (uint32_t)(chunk_pos % STAGES) * S + (uint32_t)slab;
-    return (slot >> 3) * 16384u + (slot & 7u) * 32u;
-}
+constexpr int G = SWEEP_G, RW = SWEEP_RW, WAVES = SWEEP_WAVES, S = SWEEP_S, MIN_OPS = SWEEP_MIN_OPS;
+constexpr int AHEAD = SWEEP_AHEAD, COPIES = SWEEP_COPIES;
+constexpr int VM_MARK = MIN_OPS + 1; // a marker waits until at most this many vector memory operations are under way
 } // namespace
 
 void build_sweep_plan(const int32_t *row_ptr, const int32_t *col_idx, size_t mb, size_t kb, SweepPlanHost &out)
@@ -63,7 +58,7 @@ void build_sweep_plan(const int32_t *row_ptr, const int32_t *col_idx, size_t mb,
             while (q < q_end) {
                 const int32_t bc0 = col_idx[q] / 16;
                 const int32_t cl0 = local[(size_t)bc0 / S];
-                const uint32_t off0 = lds_offset(cl0, bc0 % S);
+                const uint32_t off0 = sweep_lds_offset(cl0, bc0 % S);
                 SweepOpHost op{0, off0, 0, 0};
                 int32_t exec = cl0;
                 bool pair = false;
@@ -72,18 +67,19 @@ void build_sweep_plan(const int32_t *row_ptr, const int32_t *col_idx, size_t mb,
                     const int32_t cl1 = local[(size_t)bc1 / S];
                     if (cl1 - cl0 <= 1) { // same chunk or the next listed one: both stages are resident
                         op.w0 = (uint32_t)q * 512u;
-                        op.w2 = lds_offset(cl1, bc1 % S) - off0;
+                        op.w2 = sweep_lds_offset(cl1, bc1 % S) - off0;
                         exec = cl1;
                         pair = true;
                     }
                 }
-                if (!pair) { // both halves read the rows of B under this block; the missing half gets zeros of A
-                    if (q + 1 < nnzb) { // blocks (q, q + 1), the second multiplied by zeros
+                if (!pair) { // the other half of the MFMA reads zeros instead of rows of B
+                    if (q + 1 < nnzb) { // blocks (q, q + 1) are loaded, the second multiplies zeros
                         op.w0 = (uint32_t)q * 512u;
-                        op.w3 = OP_ZERO_HI;
-                    } else { // last block of the matrix: blocks (q - 1, q), the first multiplied by zeros
+                        op.w2 = SWEEP_ZERO_OFF - off0;
+                    } else { // last block of the matrix: blocks (q - 1, q), the first multiplies zeros
                         op.w0 = (uint32_t)(q - 1) * 512u;
-                        op.w3 = OP_ZERO_LO;
+                        op.w1 = SWEEP_ZERO_OFF;
+                        op.w2 = off0 - SWEEP_ZERO_OFF;
                     }
                 }
                 (pair ? out.n_pairs : out.n_singles)++;
@@ -138,52 +134,85 @@ void build_sweep_plan(const int32_t *row_ptr, const int32_t *col_idx, size_t mb,
             }
         }
 
-        // ---- op streams ----
+        // ---- streams: ops of chunk 0, marker, ops of chunk 1, ..., end ----
         for (int w = 0; w < WAVES; w++) {
             out.op_ptr.push_back((int32_t)out.ops.size());
+            if (n_chunks == 0) continue; // the kernel does not enter the interpreter for an empty row group
             by_chunk.assign(n_chunks, {});
             int r = 0;
             for (int lr = 0; lr < G; lr++) {
                 if (wave_of[lr] != w) continue;
                 if (r_begin + (size_t)lr < r_end) out.row_map[(rg * WAVES + (size_t)w) * RW + (size_t)r] = (int32_t)(r_begin + (size_t)lr);
                 for (const RowOp &ro : row_ops[lr]) {
-                    SweepOpHost op = ro.op;
-                    op.w3 |= (uint32_t)r * ROW_CODE << 23;
                     // rank = how many ops of this block row the chunk already holds: ops of one block
                     // row (same accumulators) end up spread over the chunk
                     int rank = 0;
                     for (const Ranked &x : by_chunk[(size_t)ro.exec]) rank += x.row == r;
-                    by_chunk[(size_t)ro.exec].push_back(Ranked{rank, r, op});
+                    by_chunk[(size_t)ro.exec].push_back(Ranked{rank, r, ro.op});
                 }
                 r++;
             }
+            struct Item { int kind, row; SweepOpHost op; }; // kind: 0 op, 1 marker, 2 end
+            std::vector<Item> items;
+            const SweepOpHost idle{0, SWEEP_ZERO_OFF, 0, 0}; // blocks 0 and 1 times zeros
             for (size_t c = 0; c < n_chunks; c++) {
                 std::vector<Ranked> &list = by_chunk[c];
                 std::stable_sort(list.begin(), list.end(), [](const Ranked &a, const Ranked &b) {
                     if (a.rank != b.rank) return a.rank < b.rank;
                     return a.row < b.row;
                 });
-                while (list.size() < (size_t)MIN_OPS) { // filler: blocks 0 and 1 times zeros, first slab of this chunk
-                    const uint32_t off = lds_offset((int32_t)c, 0);
-                    list.push_back(Ranked{0, 0, SweepOpHost{0, off, 0, OP_ZERO_HI | OP_ZERO_LO}});
+                if (c > 0) items.push_back(Item{1, 0, idle});
+                for (const Ranked &x : list) items.push_back(Item{0, x.row, x.op});
+                for (size_t k = list.size(); k < (size_t)MIN_OPS; k++) { // filler ops keep the markers AHEAD positions apart
+                    items.push_back(Item{0, 0, idle});
                     out.n_fillers++;
                 }
-                if (c > 0) list[0].op.w3 |= OP_BOUNDARY;
-                for (const Ranked &x : list) out.ops.push_back(x.op);
             }
+            items.push_back(Item{2, 0, idle});
+            // Which s_waitcnt vmcnt an op needs: vector memory operations complete in order, every position issues
+            // one A load (for the op AHEAD positions later), a marker issues its copies before that load.
+            std::vector<long> a_issue(items.size() + (size_t)AHEAD + 1, 0), copy_seq(n_chunks + 3, 0);
+            long seq = 0;
+            for (int k = 0; k < AHEAD; k++) a_issue[(size_t)k] = ++seq; // entry code, after the copies of chunks 0..2
+            size_t cur = 0;
+            for (size_t i = 0; i < items.size(); i++) {
+                Item &it = items[i];
+                if (it.kind == 2) {
+                    it.op.w3 = SWEEP_END_OFF;
+                    break;
+                }
+                if (it.kind == 1) {
+                    cur++;
+                    // the copies of chunk cur + 1 were issued by the marker before this one (or by the entry code)
+                    if (cur + 1 < n_chunks && seq - copy_seq[cur + 1] < VM_MARK) throw std::logic_error("sweep plan: a marker would not wait for its copies");
+                    if (cur + 2 < n_chunks) {
+                        seq += COPIES;
+                        copy_seq[cur + 2] = seq;
+                    }
+                    it.op.w3 = sweep_marker_code((int)i);
+                }
+                a_issue[i + (size_t)AHEAD] = ++seq;
+                if (it.kind == 0) {
+                    const long younger = seq - a_issue[i];
+                    if (younger != AHEAD && younger != AHEAD + COPIES) throw std::logic_error("sweep plan: markers closer than the A read-ahead");
+                    it.op.w3 = sweep_op_code((int)i, it.row, younger == AHEAD ? 0 : 1);
+                }
+            }
+            for (const Item &it : items) out.ops.push_back(it.op);
         }
         for (size_t c = first_chunk; c < out.chunk_ids.size(); c++) local[(size_t)out.chunk_ids[c]] = -1;
     }
     out.op_ptr.push_back((int32_t)out.ops.size());
     // what the kernel reads ahead of the last op: fetched, never executed
-    out.ops.resize(out.ops.size() + OP_PAD, SweepOpHost{0, 0, 0, OP_ZERO_HI | OP_ZERO_LO});
+    out.ops.resize(out.ops.size() + SWEEP_OP_PAD, SweepOpHost{0, SWEEP_ZERO_OFF, 0, SWEEP_END_OFF});
+    out.chunk_ids.resize(out.chunk_ids.size() + SWEEP_CHUNK_PAD, 0);
 }
 
 } // namespace smat
 
 // Test hook (not part of smat.h): builds the work list on the host and hands it out.  Arrays are
 // allocated with malloc; release each with smat_host_free.  row_map: n_rg * 64 block rows (-1 = none).  counts[0..5] = row groups, listed
-// chunks, ops (with fillers, without padding), pairs, singles, fillers.
+// chunks, stream entries (ops, fillers, markers, ends; without padding), pairs, singles, fillers.
 static int smat_internal_sweep_plan_impl(const int32_t *row_ptr, const int32_t *col_idx, size_t M, size_t K,
                                          int32_t **rg_chunk_ptr, int32_t **chunk_ids, int32_t **op_ptr,
                                          uint32_t **ops, int32_t **row_map, int64_t *counts)
@@ -208,8 +237,8 @@ static int smat_internal_sweep_plan_impl(const int32_t *row_ptr, const int32_t *
     *row_map = (int32_t *)dup(p.row_map.data(), p.row_map.size() * 4);
     if (!*rg_chunk_ptr || !*chunk_ids || !*op_ptr || !*ops || !*row_map) return SMAT_ERR_NOMEM;
     counts[0] = (int64_t)p.rg_chunk_ptr.size() - 1;
-    counts[1] = (int64_t)p.chunk_ids.size();
-    counts[2] = (int64_t)p.ops.size() - 384;
+    counts[1] = (int64_t)p.chunk_ids.size() - smat::SWEEP_CHUNK_PAD;
+    counts[2] = (int64_t)p.ops.size() - smat::SWEEP_OP_PAD;
     counts[3] = (int64_t)p.n_pairs;
     counts[4] = (int64_t)p.n_singles;
     counts[5] = (int64_t)p.n_fillers;

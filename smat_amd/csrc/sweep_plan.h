@@ -7,18 +7,18 @@
 
 #include <vector>
 
+#include "sweep_format.h"
+
 namespace smat {
 
-struct SweepOpHost { // layout: SweepOp in spmm_kernels.h
-    uint32_t w0, w1, w2, w3;
-};
+typedef SweepOp SweepOpHost; // sweep_format.h
 
 struct SweepPlanHost {
     std::vector<int32_t> rg_chunk_ptr; // n_rg + 1
-    std::vector<int32_t> chunk_ids;    // K chunk of every (row group, listed chunk)
+    std::vector<int32_t> chunk_ids;    // K chunk of every (row group, listed chunk), + SWEEP_CHUNK_PAD entries
     std::vector<int32_t> op_ptr;       // n_rg * 8 + 1
     std::vector<int32_t> row_map;      // n_rg * 64: block row of (row group, wavefront, local row), -1 = none
-    std::vector<SweepOpHost> ops;      // op streams + padding
+    std::vector<SweepOpHost> ops;      // streams (ops, markers, ends) + SWEEP_OP_PAD entries
     size_t n_pairs = 0, n_singles = 0, n_fillers = 0;
 };
 

@@ -1,9 +1,10 @@
-"""Work list of the sweep kernel, checked on the CPU: the op streams are replayed in numpy with the
-kernel's own rules (which LDS stages are resident when an op runs, at least two ops per wavefront and
-chunk, one barrier per chunk boundary in every wavefront) and the replay has to give A x B.
+"""Work list of the sweep kernel, checked on the CPU: the streams are replayed in numpy with the kernel's
+own rules and the replay has to give A x B.
 
-What the replay pins: every block is multiplied exactly once, with the rows of B under its block
-column, into its own block row; the stage an op reads holds the chunk it needs at that moment."""
+What the replay pins: every block is multiplied exactly once, with the rows of B under its block column,
+into its own block row; the LDS stage an op reads holds the chunk it needs at that moment; the code offset
+of every entry names the block of its stream position, block row and wait class; the wait class and the
+marker's wait are right for the order in which the kernel issues vector memory operations."""
 import ctypes as C
 
 import numpy as np
@@ -13,9 +14,13 @@ from smat_amd import generators as gen
 from smat_amd._lib import lib
 
 G, RW, WAVES, S, STAGES = 64, 8, 8, 16, 4
-ZERO_HI, ZERO_LO, BOUNDARY = 1, 2, 4
+AHEAD, COPIES, MIN_OPS = 3, 4, 4
+PB = 2  # the LDS reads of an op are issued this many stream positions before it
+ZERO_OFF = 131072
+BLOCK_BYTES, MARK_BASE, MARK_BYTES = 128, 16384, 512
+END_OFF = MARK_BASE + 8 * MARK_BYTES
 LDS_MASK = 0x1C0E0
-PAD = 384
+PAD, CHUNK_PAD = 16, 4
 
 
 def sweep_plan(row_ptr, col_idx, M, K):
@@ -35,10 +40,10 @@ def sweep_plan(row_ptr, col_idx, M, K):
         lib.smat_host_free(ptr)
         return a
     return {
-        "rg_chunk_ptr": take(out[0], n_rg + 1, np.int32), "chunk_ids": take(out[1], n_chunks, np.int32),
+        "rg_chunk_ptr": take(out[0], n_rg + 1, np.int32), "chunk_ids": take(out[1], n_chunks + CHUNK_PAD, np.int32),
         "op_ptr": take(out[2], n_rg * WAVES + 1, np.int32), "ops": take(out[3], (n_ops + PAD) * 4, np.uint32).reshape(-1, 4),
         "row_map": take(out[4], n_rg * G, np.int32),
-        "pairs": counts[3], "singles": counts[4], "fillers": counts[5], "n_ops": n_ops,
+        "pairs": counts[3], "singles": counts[4], "fillers": counts[5], "n_entries": n_ops,
     }
 
 
@@ -50,7 +55,7 @@ def slot_of(off):
 
 
 def replay(plan, A, Bd):
-    """Runs the op streams on dense numpy operands. A: dict from gen (BCSR), Bd: K x N float64."""
+    """Runs the streams on dense numpy operands. A: dict from gen (BCSR), Bd: K x N float64."""
     M, K, rp, ci = A["M"], A["K"], A["b_row_ptr"], A["b_col_idx"]
     blocks = A["b_val"].view(np.float16).astype(np.float64).reshape(-1, 16, 16)
     nnzb = ci.size
@@ -58,6 +63,7 @@ def replay(plan, A, Bd):
     used = np.zeros(nnzb, int)
     block_row = np.repeat(np.arange(M // 16), np.diff(rp))
     n_rg = plan["rg_chunk_ptr"].size - 1
+    n_real = n_fill = 0
     for rg in range(n_rg):
         chunks = plan["chunk_ids"][plan["rg_chunk_ptr"][rg]:plan["rg_chunk_ptr"][rg + 1]]
         assert np.all(np.diff(chunks) > 0)
@@ -66,41 +72,74 @@ def replay(plan, A, Bd):
             if chunks.size == 0:
                 assert ops.shape[0] == 0
                 continue
-            cur, in_chunk = 0, 0
-            for w0, w1, w2, w3 in ops:
-                if w3 & BOUNDARY:
-                    assert in_chunk >= 2, "fewer than two ops in a chunk"
+            # vector memory operations in issue order: the entry code loads the A operands of positions 0..AHEAD-1 after
+            # the copies of chunks 0..2; position i loads the operand of i + AHEAD, a marker issues its copies first
+            seq = AHEAD
+            a_issue = {k: k + 1 for k in range(AHEAD)}
+            copy_seq = {0: 0, 1: 0, 2: 0}
+            cur, in_chunk, ended = 0, 0, False
+            period = []  # chunk period of every stream position (a marker belongs to the chunk it opens)
+            for i, (w0, w1, w2, w3) in enumerate(tuple(int(x) for x in e) for e in ops):
+                assert not ended, "entries after the end of a stream"
+                period.append(cur + 1 if END_OFF > w3 >= MARK_BASE else cur)
+                if w3 == END_OFF:
+                    assert (w0, w1, w2) == (0, ZERO_OFF, 0)
+                    ended = True
+                    continue
+                if w3 >= MARK_BASE:
+                    assert (w3 - MARK_BASE) % MARK_BYTES == 0 and (w3 - MARK_BASE) // MARK_BYTES == i % 8
+                    assert (w0, w1, w2) == (0, ZERO_OFF, 0)
+                    assert in_chunk >= MIN_OPS, "fewer ops in a chunk than the read-ahead needs"
                     cur, in_chunk = cur + 1, 0
+                    # the marker waits until at most MIN_OPS + 1 operations are under way: its copies of the next chunk
+                    # (issued by the marker before it, or by the entry code) are older than that
+                    if cur + 1 < chunks.size:
+                        assert seq - copy_seq[cur + 1] >= MIN_OPS + 1
+                    if cur + 2 < chunks.size:
+                        seq += COPIES
+                        copy_seq[cur + 2] = seq
+                    seq += 1
+                    a_issue[i + AHEAD] = seq
+                    continue
+                seq += 1
+                a_issue[i + AHEAD] = seq
                 in_chunk += 1
-                q = int(w0) // 512
-                assert int(w0) % 512 == 0 and 0 <= q and q + 1 < nnzb and int(w3) & 0x7FFFF8 == 0
-                assert (int(w3) >> 23) % 40 == 0
-                r = (int(w3) >> 23) // 40
-                assert r < RW
+                assert w3 % BLOCK_BYTES == 0
+                k = w3 // BLOCK_BYTES
+                pos, r, v = k // 16, (k // 2) % 8, k % 2
+                assert pos == i % 8, "code block of another stream position"
+                assert seq - a_issue[i] == AHEAD + COPIES * v, "wait class does not match the operations issued since the A load"
+                q = w0 // 512
+                assert w0 % 512 == 0 and 0 <= q and q + 1 < nnzb
                 br = int(plan["row_map"][(rg * WAVES + w) * RW + r])
-                if int(w3) & (ZERO_HI | ZERO_LO) != (ZERO_HI | ZERO_LO):  # a filler may sit in a wavefront without rows
-                    assert 0 <= br < M // 16 and br // G == rg
-                off1 = (int(w1) + int(np.int32(w2))) & 0xFFFFFFFF
-                for half, (off, zero) in enumerate(((int(w1), w3 & ZERO_LO), (off1, w3 & ZERO_HI))):
-                    stage, slab = slot_of(off)
-                    # the stage holds chunk position cur or cur - 1 (whichever maps to it); cur + 1 is also
-                    # resident but no op may use it yet
-                    pos = [p for p in (cur, cur - 1) if p >= 0 and p % STAGES == stage]
-                    assert pos, "op reads a stage that holds neither its chunk nor the previous one"
-                    if zero:
+                off_lo, off_hi = w1, (w1 + int(np.int32(np.uint32(w2)))) & 0xFFFFFFFF
+                if off_lo == ZERO_OFF and off_hi == ZERO_OFF:
+                    n_fill += 1
+                    continue
+                n_real += 1
+                assert 0 <= br < M // 16 and br // G == rg
+                for half, off in enumerate((off_lo, off_hi)):
+                    if off == ZERO_OFF:
                         continue
+                    stage, slab = slot_of(off)
+                    # the stage holds chunk position cur or cur - 1 (whichever maps to it)
+                    held = [p for p in (cur, cur - 1) if p >= 0 and p % STAGES == stage]
+                    assert held, "op reads a stage that holds neither its chunk nor the previous one"
+                    # its LDS reads were issued PB positions earlier: that chunk period sees the chunks up to the next one
+                    assert held[0] <= period[max(i - PB, 0)] + 1
                     blk = q + half
-                    k0 = int(chunks[pos[0]]) * S * 16 + slab * 16
+                    k0 = int(chunks[held[0]]) * S * 16 + slab * 16
                     assert ci[blk] == k0 and block_row[blk] == br
                     used[blk] += 1
                     Cd[br * 16:br * 16 + 16] += blocks[blk] @ Bd[k0:k0 + 16]
-            assert cur == chunks.size - 1 and in_chunk >= 2
+            assert ended and cur == chunks.size - 1 and in_chunk >= MIN_OPS
     assert np.all(used == 1), "a block is multiplied zero or several times"
+    assert n_fill == plan["fillers"] and n_real == plan["pairs"] + plan["singles"]
     rows = plan["row_map"][plan["row_map"] >= 0]
     assert np.array_equal(np.sort(rows), np.arange(M // 16)), "row_map is not a partition of the block rows"
-    # read-ahead: the descriptors after the last op exist and are harmless
-    tail = plan["ops"][plan["n_ops"]:]
-    assert tail.shape[0] == PAD and np.all(tail[:, :3] == 0) and np.all(tail[:, 3] == (ZERO_HI | ZERO_LO))
+    # read-ahead: the entries after the last stream exist and are harmless
+    tail = plan["ops"][plan["n_entries"]:]
+    assert tail.shape[0] == PAD and np.all(tail == np.array([0, ZERO_OFF, 0, END_OFF], np.uint32))
     return Cd
 
 
@@ -130,7 +169,7 @@ def random_mask_matrix(mb, kb, density, seed, empty_rows=(), long_rows=()):
 
 
 @pytest.mark.parametrize("mb,kb,density,seed", [(64, 64, 0.10, 1), (70, 40, 0.30, 2), (130, 100, 0.05, 3), (8, 200, 0.5, 4),
-                                                 (64, 16, 1.0, 5), (200, 33, 0.02, 6), (3, 3, 1.0, 7)])
+                                                 (64, 16, 1.0, 5), (200, 33, 0.02, 6), (3, 3, 1.0, 7), (64, 48, 0.01, 8)])
 def test_replay_gives_a_times_b(mb, kb, density, seed):
     A = random_mask_matrix(mb, kb, density, seed, empty_rows=(1,) if mb > 2 else (), long_rows=(2,) if mb > 3 else ())
     plan = sweep_plan(A["b_row_ptr"], A["b_col_idx"], A["M"], A["K"])
@@ -139,7 +178,6 @@ def test_replay_gives_a_times_b(mb, kb, density, seed):
     Cd = replay(plan, A, Bd)
     assert np.allclose(Cd, dense_of(A) @ Bd, rtol=1e-12, atol=1e-12)
     assert plan["pairs"] * 2 + plan["singles"] == A["nnzb"]
-    assert plan["n_ops"] == plan["pairs"] + plan["singles"] + plan["fillers"]
 
 
 def test_single_last_block_is_listed_as_second_half():
@@ -151,9 +189,9 @@ def test_single_last_block_is_listed_as_second_half():
     ci = (np.nonzero(mask)[1] * 16).astype(np.int32)
     A = {"M": 32, "K": 640, "b_row_ptr": rp, "b_col_idx": ci, "b_val": gen.f16_bits(np.ones(ci.size * 256)), "nnzb": ci.size}
     plan = sweep_plan(rp, ci, 32, 640)
-    real = plan["ops"][:plan["n_ops"]]
-    lo = real[(real[:, 3] & ZERO_LO != 0) & (real[:, 3] & ZERO_HI == 0)]
-    assert lo.shape[0] == 1 and lo[0, 0] == (ci.size - 2) * 512
+    real = plan["ops"][:plan["n_entries"]]
+    lo_zero = real[(real[:, 1] == ZERO_OFF) & (real[:, 2] != 0)]  # first half reads zeros, second half a stage
+    assert lo_zero.shape[0] == 1 and lo_zero[0, 0] == (ci.size - 2) * 512
     Cd = replay(plan, A, np.ones((640, 8)))
     assert np.allclose(Cd, dense_of(A) @ np.ones((640, 8)))
 
@@ -162,7 +200,7 @@ def test_headline_matrix_pairs_nearly_everything():
     A = gen.block_pruned(8192, 0.10, 0.02)
     plan = sweep_plan(A["b_row_ptr"], A["b_col_idx"], A["M"], A["K"])
     assert plan["pairs"] * 2 + plan["singles"] == A["nnzb"]
-    # blocks paired inside a chunk or across two consecutive chunks: few stay single, hardly any filler
-    assert plan["singles"] < 0.12 * A["nnzb"] and plan["fillers"] < 0.001 * plan["n_ops"]
+    # blocks paired inside a chunk or across two consecutive chunks: few stay single, few fillers
+    assert plan["singles"] < 0.12 * A["nnzb"] and plan["fillers"] < 0.01 * (plan["pairs"] + plan["singles"])
     per_wave = np.diff(plan["op_ptr"])
-    assert per_wave.min() >= 2 * 32 and per_wave.max() <= 72 * 32
+    assert per_wave.min() >= 4 * 32 + 32 and per_wave.max() <= 72 * 32
