@@ -27,7 +27,7 @@ sys.path.insert(0, ROOT)
 PEAK_FP16_TFLOPS = 2500.0  # MI355X dense fp16 MFMA
 PEAK_HBM_GBS = 8000.0      # MI355X HBM3E
 
-KERNEL_NAMES = {1: "rowwise", 2: "sweep", 3: "rowwise", 5: "compact"}
+KERNEL_NAMES = {1: "rowwise", 2: "sweep", 3: "rowwise", 5: "compact", 6: "mixed"}
 
 
 def profiled(workload, kernel_id):
@@ -87,6 +87,10 @@ def build_workload(name):
     if name == "block_pruned_8192_10pct_N4096":
         A = gen.block_pruned(8192, 0.10, 0.02)
         N, bdist, bseed = 4096, "normal", 0xB0000004
+    elif name == "half_pruned_half_er_8192_N4096":
+        # two kinds of block rows in one matrix (dense blocks above, about one nonzero per block below): mixed dispatch
+        A = gen.half_pruned_half_er(8192, 0.10, 0.001)
+        N, bdist, bseed = 4096, "normal", 0xB0000006
     elif name == "band_4096_bw64_N128":
         d = gen.band(4096, 64)
         b = smat_amd.csr_to_bcsr(d["M"], d["K"], d["row_ptr"], d["col_idx"], d["val"])
@@ -227,7 +231,7 @@ def main():
     ap.add_argument("--steps", type=int, default=200)
     ap.add_argument("--warmup", type=int, default=20)
     ap.add_argument("--workload", default="block_pruned_8192_10pct_N4096")
-    ap.add_argument("--kernel", type=int, default=0, help="0 auto, 1 rowwise, 2 sweep, 3 rowwise reading B in place, 5 compact")
+    ap.add_argument("--kernel", type=int, default=0, help="0 auto, 1 rowwise, 2 sweep, 3 rowwise reading B in place, 5 compact, 6 mixed (rowwise + compact by block row)")
     ap.add_argument("--no-plan", action="store_true")
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--no-verify", action="store_true", help="skip the check of sampled block rows against the CPU oracle")

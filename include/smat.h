@@ -60,8 +60,13 @@ int smat_spmm_bcsr_f16(const uint16_t *vals, const int32_t *row_ptr, const int32
 
 /* ---- SpMM with options / explicit stream / plan -------------------------- */
 #define SMAT_B_COL_MAJOR 0 /* B[n*K + k]: the reference layout               */
-#define SMAT_B_ROW_MAJOR 1 /* B[k*N + n]: SMAT_KERNEL_COMPACT only (it reads rows of B; column-major B
-                            * is first copied row-major into plan scratch on every launch) */
+#define SMAT_B_ROW_MAJOR 1 /* B[k*N + n].  The compact kernel reads rows of B and takes this layout in place
+                            * (column-major B is first copied row-major into plan scratch on every launch).
+                            * The row-wise and sweep kernels feed the MFMA 8 consecutive k of one column
+                            * per lane: for them a row-major B is first transposed into the reference
+                            * layout in plan scratch (one read and one write of B per launch), which needs
+                            * a plan created with b_layout = SMAT_B_ROW_MAJOR and n_hint >= N; C has the
+                            * same bits as for column-major B */
 #define SMAT_C_F16 0       /* the reference output type                      */
 #define SMAT_C_F32 1       /* keep the fp32 accumulators                     */
 
@@ -78,6 +83,10 @@ int smat_spmm_bcsr_f16(const uint16_t *vals, const int32_t *row_ptr, const int32
 #define SMAT_KERNEL_ROWWISE_DIRECT 3 /* row-wise, B always read in place (plan or launch option)          */
 #define SMAT_KERNEL_COMPACT 5  /* only the nonzero columns of the blocks are multiplied (needs
                                * smat_plan_attach_values); for blocks with few nonzero columns */
+#define SMAT_KERNEL_MIXED 6    /* mixed dispatch inside one SpMM: block rows whose blocks are mostly full (at least
+                               * 60% of their columns nonzero) go through the row-wise kernel, the others through
+                               * the compact kernel.  Needs smat_plan_attach_values, which makes the split;
+                               * SMAT_KERNEL_AUTO takes it when each kind holds at least a tenth of the blocks */
 #define SMAT_KERNEL_ROWWISE_PACKED 4 /* row-wise, B always repacked (needs a plan created with this id) */
 
 typedef struct smat_spmm_opts {
@@ -127,10 +136,11 @@ int smat_plan_destroy(smat_plan *plan);
  * the host arrays; SMAT_ERR_INVALID when they differ.  No counterpart in the reference. */
 int smat_plan_check(const smat_plan *plan, const int32_t *row_ptr_host, const int32_t *col_idx_host,
                     size_t M, size_t K, size_t nnzb);
-/* Fills info[0..9]: kernel id, row-wise work items, split block rows, chunk size,
- * workspace bytes, panel width, sweep MFMA ops, sweep (row group, K chunk) records,
- * bytes of the scratch copy of B (0 = B is read in place), nonzero block columns listed by
- * smat_plan_attach_values (0 = not attached). */
+/* Fills info[0..11]: kernel id, row-wise work items, split block rows, chunk size,
+ * workspace bytes, panel width, sweep stream entries, sweep (row group, K chunk) records,
+ * bytes of the scratch copies of B (0 = B is read in place), nonzero block columns listed by
+ * smat_plan_attach_values (0 = not attached), and for mixed dispatch the row-wise work items and the
+ * blocks of the block rows that the row-wise kernel takes. */
 int smat_plan_info(const smat_plan *plan, int64_t *info);
 
 /* Same operands as smat_spmm_bcsr_f16; C is uint16_t* or float* per opts->c_dtype.

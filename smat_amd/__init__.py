@@ -13,6 +13,7 @@ from .host import (  # noqa: F401
     KERNEL_ROWWISE_DIRECT,
     KERNEL_ROWWISE_PACKED,
     KERNEL_COMPACT,
+    KERNEL_MIXED,
     Bcsr,
     Plan,
     csr_to_bcsr,
@@ -32,5 +33,5 @@ from .host import (  # noqa: F401
 __all__ = [
     "lib", "SmatError", "library_path", "Bcsr", "Plan", "csr_to_bcsr", "bin_write_csr", "bin_write_bcsr", "bin_read", "mtx_write", "csr_to_bcsr_device", "DeviceBcsr", "mtx_read",
     "permute_csr", "reorder_csr", "reorder_rows", "spmm",
-    "KERNEL_AUTO", "KERNEL_ROWWISE", "KERNEL_SWEEP", "KERNEL_ROWWISE_DIRECT", "KERNEL_ROWWISE_PACKED", "KERNEL_COMPACT",
+    "KERNEL_AUTO", "KERNEL_ROWWISE", "KERNEL_SWEEP", "KERNEL_ROWWISE_DIRECT", "KERNEL_ROWWISE_PACKED", "KERNEL_COMPACT", "KERNEL_MIXED",
 ]

@@ -38,15 +38,63 @@ struct smat_plan {
     size_t workspace_bytes = 0;
     uint16_t *d_bpack = nullptr; // slab-major copy of B, K * n_cap halves (row-wise kernel, when it pays)
     // sweep kernel work list (present when kernel == SMAT_KERNEL_SWEEP)
-    int n_rg = 0, n_records = 0, n_ops = 0;
-    int32_t *d_rg_chunk_ptr = nullptr, *d_chunk_ids = nullptr, *d_op_ptr = nullptr, *d_row_map = nullptr;
-    SweepOp *d_ops = nullptr;
+    struct SweepDev { // the work list of the sweep kernel in device memory
+        int n_rg = 0, n_records = 0, n_ops = 0;
+        int32_t *d_rg_chunk_ptr = nullptr, *d_chunk_ids = nullptr, *d_op_ptr = nullptr, *d_row_map = nullptr;
+        SweepOp *d_ops = nullptr;
+        hipError_t upload(const SweepPlanHost &h);
+        void release();
+        void fill(SweepArgs &w) const
+        {
+            w.rg_chunk_ptr = d_rg_chunk_ptr; w.chunk_ids = d_chunk_ids; w.op_ptr = d_op_ptr; w.ops = d_ops;
+            w.row_map = d_row_map; w.n_rg = n_rg;
+        }
+    };
+    SweepDev sweep;       // all block rows (SMAT_KERNEL_SWEEP)
+    SweepDev sweep_dense; // mixed dispatch: the block rows with mostly full blocks, when they fill the device
+    std::vector<int32_t> col_idx_host; // kept for the split of a mixed plan (plans made with col_idx_host for AUTO / MIXED)
     uint64_t fingerprint = 0; // FNV-1a over row_ptr_host and, when given, col_idx_host
     bool fingerprint_has_cols = false;
     // compacted-column kernel (present after smat_plan_attach_values)
     CompactPlan *compact = nullptr;
     uint16_t *d_bt = nullptr; // row-major copy of B, K * n_cap halves (compact kernel)
+    // mixed dispatch (after smat_plan_attach_values): row-wise work list of the block rows with mostly full blocks
+    WorkItem *d_items_dense = nullptr;
+    SplitRow *d_split_dense = nullptr;
+    float *d_workspace_dense = nullptr;
+    int n_items_dense = 0, n_split_dense = 0;
+    int64_t n_blocks_dense = 0;
+    uint16_t *d_bcol = nullptr; // column-major copy of a row-major B, K * n_cap halves (plans made for SMAT_B_ROW_MAJOR)
 };
+
+hipError_t smat_plan::SweepDev::upload(const SweepPlanHost &h)
+{
+    release();
+    n_rg = (int)h.rg_chunk_ptr.size() - 1;
+    n_records = (int)h.chunk_ids.size() - SWEEP_CHUNK_PAD;
+    n_ops = (int)(h.ops.size() - SWEEP_OP_PAD);
+    hipError_t e = hipSuccess;
+    auto up = [&](void **dst, const void *src, size_t bytes) {
+        if (e != hipSuccess) return;
+        e = hipMalloc(dst, std::max<size_t>(bytes, 16));
+        if (e == hipSuccess && bytes) e = hipMemcpy(*dst, src, bytes, hipMemcpyHostToDevice);
+    };
+    up((void **)&d_rg_chunk_ptr, h.rg_chunk_ptr.data(), h.rg_chunk_ptr.size() * sizeof(int32_t));
+    up((void **)&d_chunk_ids, h.chunk_ids.data(), h.chunk_ids.size() * sizeof(int32_t));
+    up((void **)&d_op_ptr, h.op_ptr.data(), h.op_ptr.size() * sizeof(int32_t));
+    up((void **)&d_row_map, h.row_map.data(), h.row_map.size() * sizeof(int32_t));
+    up((void **)&d_ops, h.ops.data(), h.ops.size() * sizeof(SweepOp));
+    if (e != hipSuccess) release();
+    return e;
+}
+void smat_plan::SweepDev::release()
+{
+    for (void *q : {(void *)d_rg_chunk_ptr, (void *)d_chunk_ids, (void *)d_op_ptr, (void *)d_row_map, (void *)d_ops})
+        if (q) (void)hipFree(q);
+    d_rg_chunk_ptr = d_chunk_ids = d_op_ptr = d_row_map = nullptr;
+    d_ops = nullptr;
+    n_rg = n_records = n_ops = 0;
+}
 
 extern "C" const char *smat_version(void) { return "smat-amd 0.1 gfx950"; }
 
@@ -115,7 +163,7 @@ extern "C" int smat_spmm_bcsr_f16_ex(const uint16_t *vals, const int32_t *row_pt
     if (kernel == SMAT_KERNEL_ROWWISE_PACKED && !a.b_packed)
         return set_error(SMAT_ERR_INVALID, "SMAT_KERNEL_ROWWISE_PACKED needs a plan built for it with n_hint >= N");
     if (kernel == SMAT_KERNEL_ROWWISE_DIRECT || kernel == SMAT_KERNEL_ROWWISE_PACKED) kernel = SMAT_KERNEL_ROWWISE;
-    if (kernel != SMAT_KERNEL_ROWWISE && kernel != SMAT_KERNEL_SWEEP && kernel != SMAT_KERNEL_COMPACT)
+    if (kernel != SMAT_KERNEL_ROWWISE && kernel != SMAT_KERNEL_SWEEP && kernel != SMAT_KERNEL_COMPACT && kernel != SMAT_KERNEL_MIXED)
         return set_error(SMAT_ERR_INVALID, "unknown kernel id %d", kernel);
     hipError_t e;
     if (kernel == SMAT_KERNEL_SWEEP && K >= ((size_t)1 << 28)) { // its B copies use 32-bit offsets inside four columns
@@ -126,11 +174,44 @@ extern "C" int smat_spmm_bcsr_f16_ex(const uint16_t *vals, const int32_t *row_pt
     // a plan made for a wide N, used with a narrow one: too few workgroups for the sweep kernel
     if (kernel == SMAT_KERNEL_SWEEP && o.kernel == SMAT_KERNEL_AUTO && !sweep_fills_device(M / 16, N))
         kernel = SMAT_KERNEL_ROWWISE;
-    if (o.b_layout == SMAT_B_ROW_MAJOR && kernel != SMAT_KERNEL_COMPACT)
-        return set_error(SMAT_ERR_UNSUPPORTED,
-                         "row-major B (B[k*N+n]) is implemented for SMAT_KERNEL_COMPACT only; the other kernels "
-                         "take the reference layout B[n*K+k]");
-    if (kernel == SMAT_KERNEL_COMPACT) {
+    const uint16_t *B_as_given = B;
+    if (kernel == SMAT_KERNEL_MIXED && (!plan || !plan->compact || (!plan->d_items_dense && !plan->sweep_dense.d_ops) || !plan->d_bt || N > plan->n_cap))
+        return set_error(SMAT_ERR_INVALID, "SMAT_KERNEL_MIXED needs a plan that split the block rows when the values were "
+                                           "attached (smat_plan_attach_values) and n_hint >= N");
+    if (o.b_layout == SMAT_B_ROW_MAJOR && kernel != SMAT_KERNEL_COMPACT) {
+        // the row-wise and sweep kernels want 8 consecutive k of one column in a lane: B is first brought into the
+        // reference layout in plan scratch, then they run as for column-major B (same bits in C)
+        if (!plan || !plan->d_bcol || N > plan->n_cap)
+            return set_error(SMAT_ERR_UNSUPPORTED,
+                             "row-major B (B[k*N+n]) with the row-wise or sweep kernel needs a plan created with "
+                             "b_layout = SMAT_B_ROW_MAJOR and n_hint >= N; the compact kernel reads it in place");
+        e = launch_b_to_col_major(B, plan->d_bcol, N, K, static_cast<hipStream_t>(o.stream));
+        if (e != hipSuccess) return set_error(SMAT_ERR_HIP, "SpMM launch failed: %s", hipGetErrorString(e));
+        a.B = B = plan->d_bcol;
+    }
+    if (kernel == SMAT_KERNEL_MIXED) {
+        // the block rows with mostly full blocks through the row-wise kernel, the others (and the empty ones) through
+        // the compact kernel: disjoint rows of C, one after the other on the stream
+        if (plan->sweep_dense.d_ops) {
+            SweepArgs w{};
+            w.vals = vals; w.B = B; w.C = C; w.M = M; w.N = N; w.K = K; w.nnzb = nnzb; w.c_f32 = a.c_f32;
+            plan->sweep_dense.fill(w);
+            e = launch_sweep(w, static_cast<hipStream_t>(o.stream));
+        } else {
+            SpmmArgs d = a;
+            d.items = plan->d_items_dense; d.n_items = plan->n_items_dense;
+            d.split_rows = plan->d_split_dense; d.n_split_rows = plan->n_split_dense;
+            d.workspace = plan->d_workspace_dense;
+            e = d.n_items ? launch_rowwise(d, static_cast<hipStream_t>(o.stream)) : hipSuccess;
+        }
+        if (e == hipSuccess) {
+            CompactArgs c{};
+            c.B = B_as_given; c.Bt = plan->d_bt; c.b_row_major = o.b_layout == SMAT_B_ROW_MAJOR; c.C = C; c.M = M; c.N = N; c.K = K;
+            c.c_f32 = a.c_f32;
+            c.plan = plan->compact;
+            e = launch_compact(c, static_cast<hipStream_t>(o.stream));
+        }
+    } else if (kernel == SMAT_KERNEL_COMPACT) {
         if (!plan || !plan->compact || !plan->d_bt || N > plan->n_cap)
             return set_error(SMAT_ERR_INVALID,
                              "SMAT_KERNEL_COMPACT needs a plan with attached values (smat_plan_attach_values) and n_hint >= N");
@@ -139,12 +220,11 @@ extern "C" int smat_spmm_bcsr_f16_ex(const uint16_t *vals, const int32_t *row_pt
         c.plan = plan->compact;
         e = launch_compact(c, static_cast<hipStream_t>(o.stream));
     } else if (kernel == SMAT_KERNEL_SWEEP) {
-        if (!plan || !plan->d_ops)
+        if (!plan || !plan->sweep.d_ops)
             return set_error(SMAT_ERR_INVALID, "SMAT_KERNEL_SWEEP needs a plan built for it (with col_idx_host)");
         SweepArgs w{};
         w.vals = vals; w.B = B; w.C = C; w.M = M; w.N = N; w.K = K; w.nnzb = nnzb; w.c_f32 = a.c_f32;
-        w.rg_chunk_ptr = plan->d_rg_chunk_ptr; w.chunk_ids = plan->d_chunk_ids;
-        w.op_ptr = plan->d_op_ptr; w.ops = plan->d_ops; w.row_map = plan->d_row_map; w.n_rg = plan->n_rg;
+        plan->sweep.fill(w);
         e = launch_sweep(w, static_cast<hipStream_t>(o.stream));
     } else {
         e = launch_rowwise(a, static_cast<hipStream_t>(o.stream));
@@ -226,6 +306,34 @@ static uint64_t pattern_fingerprint(const int32_t *row_ptr_host, const int32_t *
     return h;
 }
 
+// Row-wise work list: whole block rows, rows longer than `chunk` blocks in chunks with a partial-sum slot each
+// (split rows first: they are the longest items).  only != NULL: just the block rows it flags.  Returns the slots.
+static int rowwise_work_list(const int32_t *row_ptr_host, size_t mb, long chunk, const uint8_t *only,
+                             std::vector<WorkItem> &items, std::vector<SplitRow> &split)
+{
+    items.clear();
+    split.clear();
+    items.reserve(mb + 16);
+    int slot = 0;
+    for (size_t i = 0; i < mb; i++) {
+        const long len = row_ptr_host[i + 1] - row_ptr_host[i];
+        if (len <= chunk || (only && !only[i])) continue;
+        SplitRow sr{(int32_t)i, slot, slot, 0};
+        for (long b = row_ptr_host[i]; b < row_ptr_host[i + 1]; b += chunk) {
+            const long e = std::min<long>(b + chunk, row_ptr_host[i + 1]);
+            items.push_back(WorkItem{(int32_t)i, (int32_t)b, (int32_t)e, slot++});
+        }
+        sr.slot_end = slot;
+        split.push_back(sr);
+    }
+    for (size_t i = 0; i < mb; i++) {
+        const long len = row_ptr_host[i + 1] - row_ptr_host[i];
+        if (len > chunk || (only && !only[i])) continue;
+        items.push_back(WorkItem{(int32_t)i, row_ptr_host[i], row_ptr_host[i + 1], -1});
+    }
+    return slot;
+}
+
 namespace {
 struct PlanHolder { // frees a half-built plan on every way out but the good one
     smat_plan *p;
@@ -263,6 +371,7 @@ static int smat_plan_create_impl(smat_plan **out, const int32_t *row_ptr_host,
     p->kernel_requested = want;
     p->fingerprint = pattern_fingerprint(row_ptr_host, col_idx_host, mb, nnzb);
     p->fingerprint_has_cols = col_idx_host != nullptr;
+    if (col_idx_host && (want == SMAT_KERNEL_AUTO || want == SMAT_KERNEL_MIXED)) p->col_idx_host.assign(col_idx_host, col_idx_host + nnzb);
 
     // A block row is split when it is much longer than the average: chunks of
     // `chunk` blocks (even, so block pairs stay aligned with the MFMA K = 32).
@@ -276,24 +385,7 @@ static int smat_plan_create_impl(smat_plan **out, const int32_t *row_ptr_host,
 
     std::vector<WorkItem> items;
     std::vector<SplitRow> split;
-    items.reserve(mb + 16);
-    int slot = 0;
-    for (size_t i = 0; i < mb; i++) { // split rows first: they are the longest items
-        const long len = row_ptr_host[i + 1] - row_ptr_host[i];
-        if (len <= chunk) continue;
-        SplitRow sr{(int32_t)i, slot, slot, 0};
-        for (long b = row_ptr_host[i]; b < row_ptr_host[i + 1]; b += chunk) {
-            const long e = std::min<long>(b + chunk, row_ptr_host[i + 1]);
-            items.push_back(WorkItem{(int32_t)i, (int32_t)b, (int32_t)e, slot++});
-        }
-        sr.slot_end = slot;
-        split.push_back(sr);
-    }
-    for (size_t i = 0; i < mb; i++) {
-        const long len = row_ptr_host[i + 1] - row_ptr_host[i];
-        if (len > chunk) continue;
-        items.push_back(WorkItem{(int32_t)i, row_ptr_host[i], row_ptr_host[i + 1], -1});
-    }
+    const int slot = rowwise_work_list(row_ptr_host, mb, chunk, nullptr, items, split);
     p->n_items = (int)items.size();
     p->panel_tiles = rowwise_panel_tiles(n_hint, 0, items.size());
     p->n_split_rows = (int)split.size();
@@ -326,6 +418,7 @@ static int smat_plan_create_impl(smat_plan **out, const int32_t *row_ptr_host,
     // M = K in {4096, 8192, 16384}, N in {512 .. 4096} and 5% .. 25% of the blocks present: it
     // wins (by 1.02x at 5% up to 1.6x at 25%) whenever its workgroups (groups of 32 block
     // rows x panels of 128 columns) fill the 256 CUs, and loses (0.3x .. 0.9x) when they do not.
+    if (e == hipSuccess && opts && opts->b_layout == SMAT_B_ROW_MAJOR) e = hipMalloc(&p->d_bcol, K * n_hint * sizeof(uint16_t));
     bool sweep = want == SMAT_KERNEL_SWEEP;
     if (want == SMAT_KERNEL_AUTO && col_idx_host && sweep_fills_device(mb, n_hint) &&
         (double)nnzb >= 0.05 * (double)mb * (double)kb)
@@ -339,20 +432,8 @@ static int smat_plan_create_impl(smat_plan **out, const int32_t *row_ptr_host,
         SweepPlanHost h;
         build_sweep_plan(row_ptr_host, col_idx_host, mb, kb, h);
         p->kernel = SMAT_KERNEL_SWEEP;
-        p->n_rg = (int)h.rg_chunk_ptr.size() - 1;
-        p->n_records = (int)h.chunk_ids.size() - SWEEP_CHUNK_PAD;
-        p->n_ops = (int)(h.ops.size() - SWEEP_OP_PAD);
-        auto upload = [&](void **dst, const void *src, size_t bytes) {
-            if (e != hipSuccess) return;
-            e = hipMalloc(dst, std::max<size_t>(bytes, 16));
-            if (e == hipSuccess && bytes) e = hipMemcpy(*dst, src, bytes, hipMemcpyHostToDevice);
-        };
-        upload((void **)&p->d_rg_chunk_ptr, h.rg_chunk_ptr.data(), h.rg_chunk_ptr.size() * sizeof(int32_t));
-        upload((void **)&p->d_chunk_ids, h.chunk_ids.data(), h.chunk_ids.size() * sizeof(int32_t));
-        upload((void **)&p->d_op_ptr, h.op_ptr.data(), h.op_ptr.size() * sizeof(int32_t));
-        upload((void **)&p->d_row_map, h.row_map.data(), h.row_map.size() * sizeof(int32_t));
         static_assert(sizeof(SweepOpHost) == sizeof(SweepOp), "host and device op layouts");
-        upload((void **)&p->d_ops, h.ops.data(), h.ops.size() * sizeof(SweepOp));
+        e = p->sweep.upload(h);
         if (p->d_bpack && want != SMAT_KERNEL_ROWWISE_PACKED) { // the sweep kernel reads B in place
             (void)hipFree(p->d_bpack);
             p->d_bpack = nullptr;
@@ -378,34 +459,91 @@ static int smat_plan_attach_values_impl(smat_plan *p, const uint16_t *vals, cons
     if (p->nnzb && (!vals || !col_idx)) return set_error(SMAT_ERR_INVALID, "vals and col_idx must not be NULL");
     // The new list is built before the old one goes.  Whatever happens below, the old list describes values
     // that have changed, so it is dropped, and a plan left without a list goes back to a dense kernel.
+    const size_t mb = p->M / 16;
+    const int want = p->kernel_requested;
+    const bool may_mix = want == SMAT_KERNEL_AUTO || want == SMAT_KERNEL_MIXED;
+    const int dense_kernel = p->sweep.d_ops ? SMAT_KERNEL_SWEEP : SMAT_KERNEL_ROWWISE;
+    auto drop_mixed = [&] {
+        p->sweep_dense.release();
+        if (p->d_items_dense) { (void)hipFree(p->d_items_dense); p->d_items_dense = nullptr; }
+        if (p->d_split_dense) { (void)hipFree(p->d_split_dense); p->d_split_dense = nullptr; }
+        if (p->d_workspace_dense) { (void)hipFree(p->d_workspace_dense); p->d_workspace_dense = nullptr; }
+        p->n_items_dense = p->n_split_dense = 0;
+        p->n_blocks_dense = 0;
+    };
+    auto fail = [&](hipError_t err) {
+        if (p->compact) { compact_destroy(p->compact); p->compact = nullptr; }
+        drop_mixed();
+        if (p->kernel == SMAT_KERNEL_COMPACT || p->kernel == SMAT_KERNEL_MIXED) p->kernel = dense_kernel;
+        return set_error(SMAT_ERR_HIP, "attaching values failed: %s", hipGetErrorString(err));
+    };
+    // Block rows with at least 60% of their 16 x blocks columns nonzero are the dense kernels' business: they
+    // gather 16 rows of B per block, the compact kernel one row per nonzero column.  Measured: 7 nonzero columns
+    // per block (27-point stencil) 53 us compact against 86 us row-wise; 16 per block (dense blocks, N = 4096)
+    // 326 us against 180 us.  This is the per-block classification of the reference (matrix.h:400-419: blocks
+    // without / with 2:4 / with dense rows) put to use per block row.
+    std::vector<uint8_t> dense;
     CompactPlan *c = nullptr;
-    hipError_t e = compact_build(vals, row_ptr, col_idx, row_ptr_host, p->M / 16, p->nnzb, p->n_cap, &c);
-    if (p->compact) { compact_destroy(p->compact); p->compact = nullptr; }
-    const int dense_kernel = p->d_ops ? SMAT_KERNEL_SWEEP : SMAT_KERNEL_ROWWISE;
-    if (e != hipSuccess) {
-        if (p->kernel == SMAT_KERNEL_COMPACT) p->kernel = dense_kernel;
-        return set_error(SMAT_ERR_HIP, "attaching values failed: %s", hipGetErrorString(e));
+    hipError_t e = compact_build(vals, row_ptr, col_idx, row_ptr_host, mb, p->nnzb, p->n_cap, may_mix ? 0.6 : 0.0,
+                                 may_mix ? &dense : nullptr, &c);
+    if (e != hipSuccess) return fail(e);
+    int64_t blocks_dense = 0;
+    for (size_t i = 0; may_mix && i < mb; i++)
+        if (dense[i]) blocks_dense += row_ptr_host[i + 1] - row_ptr_host[i];
+    const int64_t blocks_sparse = (int64_t)p->nnzb - blocks_dense;
+    // both kinds of rows matter (a tenth of the blocks each): mixed dispatch.  Otherwise one kernel for everything.
+    bool mixed = may_mix && blocks_dense * 10 >= (int64_t)p->nnzb && blocks_sparse * 10 >= (int64_t)p->nnzb;
+    if (want == SMAT_KERNEL_MIXED) mixed = true;
+    if (may_mix && !mixed && blocks_dense > 0) { // the list left dense rows out: make it whole again
+        compact_destroy(c);
+        c = nullptr;
+        e = compact_build(vals, row_ptr, col_idx, row_ptr_host, mb, p->nnzb, p->n_cap, 0.0, nullptr, &c);
+        if (e != hipSuccess) return fail(e);
     }
-    // The dense kernels gather 16 rows of B per block, this one a row per nonzero column.  Measured:
-    // 7 nonzero columns per block (27-point stencil) 53 us against 86 us row-wise; 16 per block
-    // (dense blocks, N = 4096) 326 us against 180 us.  The plan's choice below 60% of the columns
-    // (9.6 per block), unless a kernel was asked for.
-    const bool take = p->kernel_requested == SMAT_KERNEL_COMPACT ||
-                      (p->kernel_requested == SMAT_KERNEL_AUTO && (double)c->n_cols < 0.6 * 16.0 * (double)p->nnzb);
+    if (p->compact) { compact_destroy(p->compact); p->compact = nullptr; }
+    drop_mixed();
+    const bool take = mixed || want == SMAT_KERNEL_COMPACT ||
+                      (want == SMAT_KERNEL_AUTO && (double)c->n_cols_all < 0.6 * 16.0 * (double)p->nnzb);
     if (!take) { // nothing will use the list: the plan keeps (or goes back to) a dense kernel
         compact_destroy(c);
-        if (p->kernel == SMAT_KERNEL_COMPACT) p->kernel = dense_kernel;
+        if (p->kernel == SMAT_KERNEL_COMPACT || p->kernel == SMAT_KERNEL_MIXED) p->kernel = dense_kernel;
         return SMAT_OK;
     }
     if (!p->d_bt) e = hipMalloc(&p->d_bt, p->K * p->n_cap * sizeof(uint16_t));
+    // the dense rows through the sweep kernel when their row groups of 64 fill the device, else row-wise
+    std::vector<int32_t> dense_list;
+    for (size_t i = 0; mixed && i < mb; i++)
+        if (dense[i]) dense_list.push_back((int32_t)i);
+    const bool dense_sweep = mixed && !p->col_idx_host.empty() && blocks_dense >= 2 && p->nnzb < ((size_t)1 << 23) &&
+                             p->K < ((size_t)1 << 28) && sweep_fills_device(dense_list.size(), p->n_cap);
+    if (e == hipSuccess && dense_sweep) {
+        SweepPlanHost h;
+        build_sweep_plan(row_ptr_host, p->col_idx_host.data(), mb, p->K / 16, h, dense_list.data(), dense_list.size());
+        e = p->sweep_dense.upload(h);
+        p->n_blocks_dense = blocks_dense;
+    } else if (e == hipSuccess && mixed) {
+        std::vector<WorkItem> items;
+        std::vector<SplitRow> split;
+        const int slots = rowwise_work_list(row_ptr_host, mb, p->chunk, dense.data(), items, split);
+        p->n_items_dense = (int)items.size();
+        p->n_split_dense = (int)split.size();
+        p->n_blocks_dense = blocks_dense;
+        e = hipMalloc(&p->d_items_dense, std::max<size_t>(items.size(), 1) * sizeof(WorkItem));
+        if (e == hipSuccess && !items.empty())
+            e = hipMemcpy(p->d_items_dense, items.data(), items.size() * sizeof(WorkItem), hipMemcpyHostToDevice);
+        if (e == hipSuccess && !split.empty()) {
+            e = hipMalloc(&p->d_split_dense, split.size() * sizeof(SplitRow));
+            if (e == hipSuccess) e = hipMemcpy(p->d_split_dense, split.data(), split.size() * sizeof(SplitRow), hipMemcpyHostToDevice);
+            if (e == hipSuccess) e = hipMalloc(&p->d_workspace_dense, (size_t)slots * 16 * p->n_cap * sizeof(float));
+        }
+    }
     if (e != hipSuccess) {
         compact_destroy(c);
-        if (p->kernel == SMAT_KERNEL_COMPACT) p->kernel = dense_kernel;
-        return set_error(SMAT_ERR_HIP, "attaching values failed: %s", hipGetErrorString(e));
+        return fail(e);
     }
     p->compact = c;
-    p->kernel = SMAT_KERNEL_COMPACT;
-    if (p->d_bpack && p->kernel_requested == SMAT_KERNEL_AUTO) { // the row-wise kernel's scratch is not needed any more
+    p->kernel = mixed ? SMAT_KERNEL_MIXED : SMAT_KERNEL_COMPACT;
+    if (p->d_bpack && want == SMAT_KERNEL_AUTO && !mixed) { // the row-wise kernel's scratch is not needed any more
         (void)hipFree(p->d_bpack);
         p->d_bpack = nullptr;
     }
@@ -423,15 +561,16 @@ extern "C" int smat_plan_destroy(smat_plan *p)
     if (!p) return SMAT_OK;
     if (p->compact) compact_destroy(p->compact);
     if (p->d_bt) (void)hipFree(p->d_bt);
+    if (p->d_bcol) (void)hipFree(p->d_bcol);
+    if (p->d_items_dense) (void)hipFree(p->d_items_dense);
+    if (p->d_split_dense) (void)hipFree(p->d_split_dense);
+    if (p->d_workspace_dense) (void)hipFree(p->d_workspace_dense);
     if (p->d_items) (void)hipFree(p->d_items);
     if (p->d_split) (void)hipFree(p->d_split);
     if (p->d_workspace) (void)hipFree(p->d_workspace);
     if (p->d_bpack) (void)hipFree(p->d_bpack);
-    if (p->d_rg_chunk_ptr) (void)hipFree(p->d_rg_chunk_ptr);
-    if (p->d_chunk_ids) (void)hipFree(p->d_chunk_ids);
-    if (p->d_op_ptr) (void)hipFree(p->d_op_ptr);
-    if (p->d_row_map) (void)hipFree(p->d_row_map);
-    if (p->d_ops) (void)hipFree(p->d_ops);
+    p->sweep.release();
+    p->sweep_dense.release();
     delete p;
     return SMAT_OK;
 }
@@ -456,10 +595,12 @@ extern "C" int smat_plan_info(const smat_plan *p, int64_t *info)
     info[0] = p->kernel; info[1] = p->n_items; info[2] = p->n_split_rows; info[3] = p->chunk;
     info[4] = (int64_t)p->workspace_bytes;
     info[5] = p->kernel == SMAT_KERNEL_SWEEP ? 16 * SWEEP_TN : 16 * p->panel_tiles;
-    info[6] = p->n_ops; info[7] = p->n_records;
+    info[6] = p->sweep.n_ops + p->sweep_dense.n_ops; info[7] = p->sweep.n_records + p->sweep_dense.n_records;
     info[8] = (p->d_bpack ? (int64_t)(p->K * p->n_cap * sizeof(uint16_t)) : 0) +
-              (p->d_bt ? (int64_t)(p->K * p->n_cap * sizeof(uint16_t)) : 0);
+              (p->d_bt ? (int64_t)(p->K * p->n_cap * sizeof(uint16_t)) : 0) +
+              (p->d_bcol ? (int64_t)(p->K * p->n_cap * sizeof(uint16_t)) : 0);
     info[9] = p->compact ? p->compact->n_cols : 0;
+    info[10] = p->n_items_dense; info[11] = p->n_blocks_dense;
     return SMAT_OK;
 }
 

@@ -46,7 +46,7 @@ public:
             // the plan also looks at the block values once (which columns of the blocks are nonzero)
             SMAT_CHECK(smat_plan_attach_values(plan_, (const uint16_t *)A_->getBcsrValues(), A_->getBcsrRowPtr(),
                                                A_->getBcsrColIdx(), A_->hostBcsrRowPtr()));
-            int64_t info[10];
+            int64_t info[12];
             SMAT_CHECK(smat_plan_info(plan_, info));
             HLOG("Plan: kernel %lld, %lld work items, %lld split block rows, workspace %lld bytes, %lld sweep ops, "
                  "%lld nonzero block columns",

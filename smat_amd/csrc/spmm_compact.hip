@@ -102,6 +102,7 @@ __global__ void gather_kernel(const uint16_t *__restrict__ vals, const uint16_t 
         const long mid = (lo + hi) >> 1;
         if (row_ptr[mid] <= p) lo = mid; else hi = mid;
     }
+    if (padded_start[lo] < 0) return; // a block row that another kernel multiplies
     long o = (long)padded_start[lo] + (offset[p] - offset[row_ptr[lo]]);
     const int32_t c0 = col_idx[p];
     const uint16_t *blk = vals + p * 256;
@@ -320,6 +321,15 @@ struct Scratch {
 
 } // namespace
 
+// Row-major B (B[k*N + n]) -> column-major out[n*K + k]: the same tile transposition with the roles of the
+// two dimensions swapped (N % 8 == 0 and K % 16 == 0 keep every 16-byte access aligned).
+hipError_t launch_b_to_col_major(const uint16_t *B_row_major, uint16_t *out, size_t N, size_t K, hipStream_t st)
+{
+    dim3 grid((unsigned)((N + 63) / 64), (unsigned)((K + 63) / 64));
+    hipLaunchKernelGGL(transpose_b_kernel, grid, dim3(256), 0, st, B_row_major, out, (int)K, (long)N);
+    return hipGetLastError();
+}
+
 hipError_t launch_compact(const CompactArgs &a_in, hipStream_t st)
 {
     CompactArgs a = a_in;
@@ -355,7 +365,8 @@ void compact_destroy(CompactPlan *p)
 }
 
 hipError_t compact_build(const uint16_t *vals, const int32_t *row_ptr, const int32_t *col_idx,
-                         const int32_t *row_ptr_host, size_t mb, size_t nnzb, size_t n_cap, CompactPlan **out)
+                         const int32_t *row_ptr_host, size_t mb, size_t nnzb, size_t n_cap, double dense_share,
+                         std::vector<uint8_t> *dense_rows, CompactPlan **out)
 {
     *out = nullptr;
     CompactPlan *p = new (std::nothrow) CompactPlan();
@@ -389,22 +400,37 @@ hipError_t compact_build(const uint16_t *vals, const int32_t *row_ptr, const int
         SMAT_STEP(hipMemcpy(raw.data(), cc.p, (mb + 1) * 4, hipMemcpyDeviceToHost));
         n_cols = raw[mb];
     }
+    // Block rows whose blocks are mostly full (at least dense_share of their 16 x blocks columns are nonzero) are
+    // left to a dense kernel when the caller asks for the split: they get no list and no work item here.
+    std::vector<uint8_t> dense(mb, 0);
+    p->n_cols_all = n_cols;
+    if (dense_rows && dense_share > 0.0)
+        for (size_t i = 0; i < mb; i++) {
+            const int64_t blocks = row_ptr_host[i + 1] - row_ptr_host[i];
+            if (blocks > 0 && (double)(raw[i + 1] - raw[i]) >= dense_share * 16.0 * (double)blocks) {
+                dense[i] = 1;
+                n_cols -= raw[i + 1] - raw[i];
+            }
+        }
     p->n_cols = n_cols;
     // every block row is padded to a multiple of 32 columns (one MFMA step); padding = zero columns
     int64_t total = 0;
+    std::vector<int32_t> padded_dev(mb + 1, 0); // what the gather kernel sees: -1 for rows without a list
     for (size_t i = 0; i < mb; i++) {
         padded[i] = (int32_t)total;
-        total += ((int64_t)(raw[i + 1] - raw[i]) + 31) / 32 * 32;
+        padded_dev[i] = dense[i] ? -1 : (int32_t)total;
+        if (!dense[i]) total += ((int64_t)(raw[i + 1] - raw[i]) + 31) / 32 * 32;
         if (total > 0x7fffff00) e = hipErrorInvalidValue;
     }
     padded[mb] = (int32_t)total;
+    padded_dev[mb] = (int32_t)total;
     const size_t cap = (size_t)total + LIST_PAD;
     SMAT_STEP(hipMalloc(&p->d_cols, cap * sizeof(int32_t)));
     SMAT_STEP(hipMemset(p->d_cols, 0, cap * sizeof(int32_t))); // padding: row 0 of B
     SMAT_STEP(hipMalloc(&p->d_acol, cap * 16 * sizeof(uint16_t)));
     SMAT_STEP(hipMemset(p->d_acol, 0, cap * 16 * sizeof(uint16_t)));
     if (e == hipSuccess && nnzb) {
-        SMAT_STEP(hipMemcpy(cc.p, padded.data(), (mb + 1) * 4, hipMemcpyHostToDevice));
+        SMAT_STEP(hipMemcpy(cc.p, padded_dev.data(), (mb + 1) * 4, hipMemcpyHostToDevice));
         if (e == hipSuccess) {
             hipLaunchKernelGGL(gather_kernel, dim3((unsigned)((nnzb + 255) / 256)), dim3(256), 0, 0, vals,
                                (const uint16_t *)mask.p, (const int32_t *)offset.p, row_ptr, col_idx,
@@ -413,7 +439,6 @@ hipError_t compact_build(const uint16_t *vals, const int32_t *row_ptr, const int
         }
     }
     // work items: whole block rows; rows much longer than the average in chunks of 32-column steps
-    (void)row_ptr_host;
     const std::vector<int32_t> &cc_host = padded;
     size_t nonempty = 0;
     for (size_t i = 0; i < mb; i++) nonempty += cc_host[i + 1] > cc_host[i];
@@ -426,7 +451,7 @@ hipError_t compact_build(const uint16_t *vals, const int32_t *row_ptr, const int
     int slot = 0;
     for (size_t i = 0; i < mb; i++) {
         const long len = cc_host[i + 1] - cc_host[i];
-        if (len <= chunk) continue;
+        if (len <= chunk || dense[i]) continue;
         SplitRow sr{(int32_t)i, slot, slot, 0};
         for (long b = cc_host[i]; b < cc_host[i + 1]; b += chunk)
             items.push_back(WorkItem{(int32_t)i, (int32_t)b, (int32_t)std::min<long>(b + chunk, cc_host[i + 1]), slot++});
@@ -435,9 +460,10 @@ hipError_t compact_build(const uint16_t *vals, const int32_t *row_ptr, const int
     }
     for (size_t i = 0; i < mb; i++) {
         const long len = cc_host[i + 1] - cc_host[i];
-        if (len > chunk) continue;
+        if (len > chunk || dense[i]) continue;
         items.push_back(WorkItem{(int32_t)i, cc_host[i], cc_host[i + 1], -1});
     }
+    if (dense_rows) *dense_rows = dense;
     p->n_items = (int)items.size();
     p->n_split_rows = (int)split.size();
     p->n_slots = slot;

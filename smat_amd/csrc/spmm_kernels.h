@@ -3,6 +3,7 @@
 #include <hip/hip_runtime.h>
 
 #include "sweep_format.h"
+#include <vector>
 #include <stddef.h>
 #include <stdint.h>
 
@@ -72,11 +73,15 @@ struct CompactPlan {
     SplitRow *d_split = nullptr;
     float *d_workspace = nullptr; // n_slots * 16 * n_cap floats
     int n_items = 0, n_split_rows = 0, n_slots = 0;
-    int64_t n_cols = 0;           // nonzero block columns (without padding)
+    int64_t n_cols = 0;           // nonzero block columns listed (without padding)
+    int64_t n_cols_all = 0;       // nonzero block columns of the whole matrix
 };
 // vals / row_ptr / col_idx: device BCSR arrays; row_ptr_host: host copy of row_ptr.
+// dense_rows != NULL and dense_share > 0: block rows with at least that share of nonzero columns get no list and no
+// work item (a dense kernel multiplies them); *dense_rows receives one flag per block row.
 hipError_t compact_build(const uint16_t *vals, const int32_t *row_ptr, const int32_t *col_idx,
-                         const int32_t *row_ptr_host, size_t mb, size_t nnzb, size_t n_cap, CompactPlan **out);
+                         const int32_t *row_ptr_host, size_t mb, size_t nnzb, size_t n_cap, double dense_share,
+                         std::vector<uint8_t> *dense_rows, CompactPlan **out);
 void compact_destroy(CompactPlan *p);
 struct CompactArgs {
     const uint16_t *B; // column-major, or row-major with b_row_major
@@ -88,6 +93,7 @@ struct CompactArgs {
     const CompactPlan *plan;
 };
 hipError_t launch_compact(const CompactArgs &a, hipStream_t st);
+hipError_t launch_b_to_col_major(const uint16_t *B_row_major, uint16_t *out, size_t N, size_t K, hipStream_t st);
 
 int rowwise_panel_tiles(size_t N, int requested, size_t n_items);
 hipError_t launch_sweep(const SweepArgs &a, hipStream_t st);

@@ -19,9 +19,12 @@ constexpr int AHEAD = SWEEP_AHEAD, COPIES = SWEEP_COPIES;
 constexpr int VM_MARK = MIN_OPS + 1; // a marker waits until at most this many vector memory operations are under way
 } // namespace
 
-void build_sweep_plan(const int32_t *row_ptr, const int32_t *col_idx, size_t mb, size_t kb, SweepPlanHost &out)
+void build_sweep_plan(const int32_t *row_ptr, const int32_t *col_idx, size_t mb, size_t kb, SweepPlanHost &out,
+                      const int32_t *rows, size_t n_rows)
 {
-    const size_t n_rg = (mb + G - 1) / G;
+    if (!rows) n_rows = mb;
+    auto row_at = [&](size_t i) { return rows ? (size_t)rows[i] : i; }; // i-th block row of the plan
+    const size_t n_rg = (n_rows + G - 1) / G;
     const size_t n_kchunks = (kb + S - 1) / S;
     const int32_t nnzb = row_ptr[mb];
     out = SweepPlanHost();
@@ -35,10 +38,11 @@ void build_sweep_plan(const int32_t *row_ptr, const int32_t *col_idx, size_t mb,
     std::vector<std::vector<Ranked>> by_chunk;
     std::vector<int32_t> count; // ops of (row, chunk)
     for (size_t rg = 0; rg < n_rg; rg++) {
-        const size_t r_begin = rg * G, r_end = std::min(mb, (rg + 1) * G);
+        const size_t r_begin = rg * G, r_end = std::min(n_rows, (rg + 1) * G);
         // the chunks this row group touches, ascending
         const size_t first_chunk = out.chunk_ids.size();
-        for (int32_t q = row_ptr[r_begin]; q < row_ptr[r_end]; q++) local[(size_t)(col_idx[q] / 16) / S] = 0;
+        for (size_t i = r_begin; i < r_end; i++)
+            for (int32_t q = row_ptr[row_at(i)]; q < row_ptr[row_at(i) + 1]; q++) local[(size_t)(col_idx[q] / 16) / S] = 0;
         for (size_t c = 0; c < n_kchunks; c++)
             if (local[c] == 0) {
                 local[c] = (int32_t)(out.chunk_ids.size() - first_chunk);
@@ -51,8 +55,8 @@ void build_sweep_plan(const int32_t *row_ptr, const int32_t *col_idx, size_t mb,
         count.assign((size_t)G * std::max<size_t>(n_chunks, 1), 0);
         for (int lr = 0; lr < G; lr++) {
             row_ops[lr].clear();
-            const size_t br = r_begin + (size_t)lr;
-            if (br >= r_end) continue;
+            if (r_begin + (size_t)lr >= r_end) continue;
+            const size_t br = row_at(r_begin + (size_t)lr);
             int32_t q = row_ptr[br];
             const int32_t q_end = row_ptr[br + 1];
             while (q < q_end) {
@@ -142,7 +146,7 @@ void build_sweep_plan(const int32_t *row_ptr, const int32_t *col_idx, size_t mb,
             int r = 0;
             for (int lr = 0; lr < G; lr++) {
                 if (wave_of[lr] != w) continue;
-                if (r_begin + (size_t)lr < r_end) out.row_map[(rg * WAVES + (size_t)w) * RW + (size_t)r] = (int32_t)(r_begin + (size_t)lr);
+                if (r_begin + (size_t)lr < r_end) out.row_map[(rg * WAVES + (size_t)w) * RW + (size_t)r] = (int32_t)row_at(r_begin + (size_t)lr);
                 for (const RowOp &ro : row_ops[lr]) {
                     // rank = how many ops of this block row the chunk already holds: ops of one block
                     // row (same accumulators) end up spread over the chunk

@@ -23,7 +23,9 @@ struct SweepPlanHost {
 };
 
 // row_ptr / col_idx: host BCSR (col_idx = absolute first column of each block, validated by the caller);
-// at least two blocks.
-void build_sweep_plan(const int32_t *row_ptr, const int32_t *col_idx, size_t mb, size_t kb, SweepPlanHost &out);
+// at least two blocks.  rows != NULL: only these n_rows block rows (ascending) are multiplied and stored, packed
+// 64 to a row group; the others belong to another kernel.
+void build_sweep_plan(const int32_t *row_ptr, const int32_t *col_idx, size_t mb, size_t kb, SweepPlanHost &out,
+                      const int32_t *rows = nullptr, size_t n_rows = 0);
 
 } // namespace smat

@@ -130,6 +130,24 @@ def block_pruned(M=8192, keep=0.10, sigma=0.02, seed=0x5A170004):
     return {"M": M, "K": M, "b_row_ptr": row_ptr, "b_col_idx": col_idx, "b_val": val, "nnzb": kept}
 
 
+def half_pruned_half_er(M=8192, keep=0.10, density=0.001, seed=0x5A170006):
+    """A matrix of two kinds of rows: the upper half of its block rows from block_pruned (dense 16x16 blocks), the
+    lower half the blocking of an Erdos-Renyi matrix (about one nonzero per block).  BCSR arrays like block_pruned."""
+    from . import host
+    mb = M // 16
+    top = block_pruned(M, keep, 0.02, seed)
+    er = erdos_renyi(M, density, seed ^ 0x77)
+    low = host.csr_to_bcsr(er["M"], er["K"], er["row_ptr"], er["col_idx"], er["val"])
+    h = mb // 2
+    t_end = int(top["b_row_ptr"][h])
+    l_begin = int(low.row_ptr[h])
+    row_ptr = np.concatenate([top["b_row_ptr"][:h + 1], low.row_ptr[h + 1:] - l_begin + t_end]).astype(np.int32)
+    col_idx = np.concatenate([top["b_col_idx"][:t_end], low.col_idx[l_begin:]]).astype(np.int32)
+    val = np.concatenate([top["b_val"][:t_end * 256], low.val[l_begin * 256:]])
+    return {"M": M, "K": M, "b_row_ptr": row_ptr, "b_col_idx": col_idx, "b_val": val, "nnzb": int(col_idx.size),
+            "dense_blocks": t_end}
+
+
 def bcsr_to_csr(M, b_row_ptr, b_col_idx, b_val, drop_zeros=False):
     """Expands BCSR blocks to a CSR (all 256 entries per block unless drop_zeros)."""
     mb = M // 16

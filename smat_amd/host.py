@@ -12,6 +12,7 @@ from ._lib import SpmmOpts, check, lib
 
 BS = 16
 KERNEL_AUTO, KERNEL_ROWWISE, KERNEL_SWEEP, KERNEL_ROWWISE_DIRECT, KERNEL_ROWWISE_PACKED, KERNEL_COMPACT = 0, 1, 2, 3, 4, 5
+KERNEL_MIXED = 6
 C_F16, C_F32 = 0, 1
 
 
@@ -209,11 +210,11 @@ def permute_csr(M, K, row_ptr, col_idx, val, perm_rows=None, perm_cols=None):
 class Plan:
     """Per-matrix work list (built once, outside any timed loop)."""
 
-    def __init__(self, row_ptr_host, M, K, nnzb, n_hint, col_idx_host=None, kernel=KERNEL_AUTO):
+    def __init__(self, row_ptr_host, M, K, nnzb, n_hint, col_idx_host=None, kernel=KERNEL_AUTO, b_row_major=False):
         self._h = C.c_void_p()
         rp = np.ascontiguousarray(row_ptr_host, dtype=np.int32)
         ci = None if col_idx_host is None else np.ascontiguousarray(col_idx_host, dtype=np.int32)
-        opts = SpmmOpts(0, 0, kernel, 0, None)
+        opts = SpmmOpts(1 if b_row_major else 0, 0, kernel, 0, None)
         check(lib.smat_plan_create(C.byref(self._h), _p(rp), _p(ci), M, K, nnzb, n_hint, C.byref(opts)))
         self._rp_host = rp
 
@@ -233,10 +234,10 @@ class Plan:
         return self._h
 
     def info(self):
-        out = (C.c_int64 * 10)()
+        out = (C.c_int64 * 12)()
         check(lib.smat_plan_info(self._h, out))
         keys = ("kernel", "items", "split_rows", "chunk", "workspace_bytes", "panel", "sweep_ops", "sweep_records",
-                "b_pack_bytes", "compact_cols")
+                "b_pack_bytes", "compact_cols", "mixed_dense_items", "mixed_dense_blocks")
         return dict(zip(keys, out))
 
     def close(self):

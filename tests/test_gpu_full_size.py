@@ -120,3 +120,17 @@ def test_config5_stencil_64_full_size(smat, cuda, oracle, reordered):
     C1, _ = gpu_spmm_compact(smat, cuda, A, B, N, kernel=1)
     a, b = C.view(np.float16).astype(np.float32), C1.view(np.float16).astype(np.float32)
     assert np.abs(a - b).max() <= 2e-3 * np.abs(b).max()
+
+
+def test_mixed_dispatch_full_size(smat, cuda, oracle):
+    """8192 x 8192, upper half of the block rows dense blocks (10 % kept), lower half about one nonzero per
+    block, N = 4096: the plan sends the upper half through the sweep kernel (its 256 block rows fill the device)
+    and the lower half through the compact kernel."""
+    A = gen.half_pruned_half_er(8192, 0.10, 0.001)
+    N = 4096
+    B = gen.dense_b(A["K"], N, seed=0xB0000006, dist="normal")
+    C, info = gpu_spmm_compact(smat, cuda, A, B, N, kernel=0)
+    assert info["kernel"] == 6 and info["mixed_dense_blocks"] == A["dense_blocks"]
+    assert info["sweep_ops"] > 0 and info["mixed_dense_items"] == 0  # sweep, not row-wise, for the dense rows
+    mb = A["M"] // 16
+    check_sampled(oracle, A, B, N, C, sample_rows(mb, 16, extra=(mb // 2 - 1, mb // 2, mb // 2 + 1)))

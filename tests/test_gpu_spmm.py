@@ -444,10 +444,31 @@ def test_compact_kernel_row_major_b(smat, cuda, oracle):
         out.append(C.cpu().numpy().view(np.uint16))
     assert np.array_equal(out[0], out[1])
     assert oracle.compare(out[0], oracle_ref(oracle, A, B, N))[0] <= TOL_F16
-    with pytest.raises(smat.SmatError, match="row-major"):
+    with pytest.raises(smat.SmatError, match="row-major"):  # the dense kernels need a plan made for row-major B
         C = torch.zeros((M, N), dtype=torch.int16, device=cuda)
         smat.spmm(vals, rp, ci, to_dev(torch, B_rm, cuda), C, M, N, K, nnzb, plan=p, kernel=1, b_row_major=True)
     p.close()
+
+
+@pytest.mark.parametrize("kernel", [1, 2, 3, 4])
+def test_row_major_b_dense_kernels_bit_identical(smat, cuda, oracle, kernel):
+    """Row-major B with the row-wise and sweep kernels: the same bits as the reference layout gives."""
+    import torch
+    A = gen.random_bcsr(70, 45, 0.2, seed=77)
+    M, K, nnzb, N = A["M"], A["K"], A["nnzb"], 136
+    B = gen.dense_b(K, N, seed=78, dist="normal")
+    B_rm = np.ascontiguousarray(B.reshape(N, K).T).ravel()
+    vals, rp, ci = to_dev(torch, A["b_val"], cuda), to_dev(torch, A["b_row_ptr"].astype(np.int32), cuda), to_dev(torch, A["b_col_idx"].astype(np.int32), cuda)
+    out = []
+    for bits, rm in ((B, False), (B_rm, True)):
+        p = smat.Plan(A["b_row_ptr"], M, K, nnzb, N, col_idx_host=A["b_col_idx"], kernel=kernel, b_row_major=rm)
+        C = torch.full((M, N), 0x7E00, dtype=torch.int16, device=cuda)
+        smat.spmm(vals, rp, ci, to_dev(torch, bits, cuda), C, M, N, K, nnzb, plan=p, kernel=kernel, b_row_major=rm)
+        torch.cuda.synchronize()
+        out.append(C.cpu().numpy().view(np.uint16))
+        p.close()
+    assert np.array_equal(out[0], out[1])
+    assert oracle.compare(out[0], oracle_ref(oracle, A, B, N))[0] <= TOL_F16
 
 
 def test_compact_kernel_config2_full_size(smat, cuda, oracle):
@@ -503,3 +524,46 @@ def test_plan_check_tells_patterns_apart(smat, cuda):
         with pytest.raises(smat.SmatError, match="another block pattern"):
             plan.check(rp2, None, A["M"], A["K"], nnzb)
     plan.close()
+
+
+MIXED = 6
+
+
+def test_mixed_dispatch_half_dense_half_sparse_rows(smat, cuda, oracle):
+    """Half the block rows hold dense blocks, half about one nonzero per block: the plan splits them at attach
+    time, the row-wise kernel takes the first kind, the compact kernel the second, and C is whole."""
+    A = gen.half_pruned_half_er(2048, 0.15, 0.004, seed=91)
+    M, K, nnzb = A["M"], A["K"], A["nnzb"]
+    N = 264
+    B = gen.dense_b(K, N, seed=92, dist="normal")
+    ref = oracle_ref(oracle, A, B, N)
+    C, info = gpu_spmm_compact(smat, cuda, A, B, N, kernel=0)       # the plan's own choice
+    assert info["kernel"] == MIXED
+    assert info["mixed_dense_blocks"] == A["dense_blocks"] and 0 < info["mixed_dense_items"] <= M // 32 + 8
+    assert 0 < info["compact_cols"] < 3 * (nnzb - A["dense_blocks"])  # the list holds the sparse rows only
+    assert oracle.compare(C, ref)[0] <= TOL_F16
+    C32, _ = gpu_spmm_compact(smat, cuda, A, B, N, kernel=MIXED, c_f32=True)
+    assert rel_err_f32(C32, ref) <= TOL_F32
+    # each single kernel on the same matrix: same tolerance, and the rows each kernel of the mixed plan wrote
+    # carry exactly the bits that kernel writes alone (same work items, same arithmetic)
+    C_row, _ = gpu_spmm_compact(smat, cuda, A, B, N, kernel=1)
+    C_cmp, _ = gpu_spmm_compact(smat, cuda, A, B, N, kernel=COMPACT)
+    half = M // 2
+    assert np.array_equal(C[:half], C_row[:half]) and np.array_equal(C[half:], C_cmp[half:])
+
+
+def test_mixed_dispatch_falls_back_to_one_kernel(smat, cuda, oracle):
+    """All rows of one kind: the plan keeps a single kernel (compact for sparse blocks, a dense one for full blocks)."""
+    d = gen.erdos_renyi(1024, 0.004, seed=5)
+    A = bcsr_of(smat, d)
+    B = gen.dense_b(A["K"], 64, seed=6, dist="uniform")
+    C, info = gpu_spmm_compact(smat, cuda, A, B, 64, kernel=0)
+    assert info["kernel"] == COMPACT and info["mixed_dense_items"] == 0
+    assert oracle.compare(C, oracle_ref(oracle, A, B, 64))[0] <= TOL_F16
+    A = gen.random_bcsr(40, 40, 0.2, seed=7)
+    B = gen.dense_b(A["K"], 64, seed=8, dist="uniform")
+    C, info = gpu_spmm_compact(smat, cuda, A, B, 64, kernel=0)
+    assert info["kernel"] in (1, 2) and info["compact_cols"] == 0
+    assert oracle.compare(C, oracle_ref(oracle, A, B, 64))[0] <= TOL_F16
+    with pytest.raises(smat.SmatError, match="SMAT_KERNEL_MIXED needs a plan"):
+        gpu_spmm(smat, cuda, A, B, 64, plan=True, kernel=MIXED)
