@@ -146,11 +146,14 @@ int smat_plan_info(const smat_plan *plan, int64_t *info);
 /* Same operands as smat_spmm_bcsr_f16; C is uint16_t* or float* per opts->c_dtype.
  * opts == NULL means defaults; plan == NULL means no work list (whole block
  * rows, one wavefront each).
- * Non-finite inputs: an unpaired block is multiplied together with a block of zeros
- * (one MFMA covers two blocks) and the compact kernel pads a block row with zero
- * columns; 0 x Inf = NaN, so where B holds Inf or NaN a result element can come out
- * NaN where a block-by-block product (mmaCBT.cu:44-66) gives Inf.  Finite inputs give
- * the same sums up to the fp32 summation order. */
+ * Non-finite inputs: one MFMA covers two blocks.  The row-wise kernel multiplies an unpaired
+ * block together with a block of zeros, the compact kernel pads a block row with zero columns
+ * (0 x Inf = NaN where B holds Inf or NaN).  The sweep kernel multiplies an unpaired block together
+ * with the block that follows it in vals (the one before it for the last block) and 16 rows of zeros
+ * in place of B, and its filler ops multiply blocks 0 and 1 by zeros: where vals holds Inf or NaN, a
+ * row of C that another block row's block shares an MFMA with can come out NaN.  A block-by-block
+ * product (mmaCBT.cu:44-66) gives Inf / NaN only where the operands of that element hold them.
+ * Finite inputs give the same sums up to the fp32 summation order. */
 int smat_spmm_bcsr_f16_ex(const uint16_t *vals, const int32_t *row_ptr, const int32_t *col_idx,
                           const uint16_t *B, void *C, size_t M, size_t N, size_t K, size_t nnzb,
                           const smat_spmm_opts *opts, const smat_plan *plan);
