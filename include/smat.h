@@ -130,6 +130,12 @@ int smat_plan_create(smat_plan **plan, const int32_t *row_ptr_host, const int32_
  * 16x16 (mmaCBT.cu:44-66). */
 int smat_plan_attach_values(smat_plan *plan, const uint16_t *vals, const int32_t *row_ptr,
                             const int32_t *col_idx, const int32_t *row_ptr_host);
+/* Staleness guard for the copy that smat_plan_attach_values keeps: *current = 1 when the block values in vals
+ * (device) still have the checksum they had when they were attached (or when no kernel of the plan works from
+ * a copy), 0 when they have changed and must be attached again.  One pass over vals at memory speed plus an
+ * 8-byte copy back (synchronous): 3 us for 13 MB of values, 1.3 ms for the 5.7 GB of R-MAT scale 20.  Not
+ * called by the SpMM itself.  No counterpart in the reference, which keeps no copy. */
+int smat_plan_values_current(const smat_plan *plan, const uint16_t *vals, int *current);
 int smat_plan_destroy(smat_plan *plan);
 /* Opt-in check that `plan` was made from this block pattern: M, K, nnzb and a 64-bit FNV-1a hash of
  * row_ptr_host (and of col_idx_host if the plan was made with one; then it must be passed).  One pass over

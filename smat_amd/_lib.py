@@ -37,6 +37,7 @@ SIGNATURES = {
     "smat_spmm_bcsr_f16": (_int, [_vp, _vp, _vp, _vp, _vp, _sz, _sz, _sz, _sz, _vp, _vp]),
     "smat_spmm_bcsr_f16_ex": (_int, [_vp, _vp, _vp, _vp, _vp, _sz, _sz, _sz, _sz, C.POINTER(SpmmOpts), _vp]),
     "smat_spmm_bcsr_f16_static": (_int, [_vp, _vp, _vp, _vp, _vp, _sz, _sz, _sz, _sz, _vp]),
+    "smat_plan_values_current": (_int, [_vp, _vp, C.POINTER(C.c_int)]),
     "smat_plan_check": (_int, [_vp, _vp, _vp, _sz, _sz, _sz]),
     "smat_plan_create": (_int, [_pp, _vp, _vp, _sz, _sz, _sz, _sz, C.POINTER(SpmmOpts)]),
     "smat_plan_attach_values": (_int, [_vp, _vp, _vp, _vp, _vp]),

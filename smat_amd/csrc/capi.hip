@@ -589,6 +589,19 @@ extern "C" int smat_plan_check(const smat_plan *p, const int32_t *row_ptr_host, 
     return SMAT_OK;
 }
 
+extern "C" int smat_plan_values_current(const smat_plan *p, const uint16_t *vals, int *current)
+{
+    if (!p || !current) return set_error(SMAT_ERR_INVALID, "plan and current must not be NULL");
+    *current = 1;
+    if (!p->compact) return SMAT_OK; // no kernel of this plan works from a copy of the values
+    if (p->nnzb && !vals) return set_error(SMAT_ERR_INVALID, "vals must not be NULL");
+    uint64_t h = 0;
+    hipError_t e = values_checksum(vals, p->nnzb, &h);
+    if (e != hipSuccess) return set_error(SMAT_ERR_HIP, "checksum of the block values failed: %s", hipGetErrorString(e));
+    *current = h == p->compact->values_checksum;
+    return SMAT_OK;
+}
+
 extern "C" int smat_plan_info(const smat_plan *p, int64_t *info)
 {
     if (!p || !info) return set_error(SMAT_ERR_INVALID, "plan and info must not be NULL");

@@ -86,6 +86,18 @@ __global__ __launch_bounds__(256) void colmask_kernel(const uint16_t *__restrict
     }
 }
 
+// Order-independent 64-bit checksum of the block values: sum over all dwords of value * (2 * index + 1).
+__global__ __launch_bounds__(256) void values_checksum_kernel(const uint32_t *__restrict__ vals, long n_dwords,
+                                                              unsigned long long *__restrict__ out)
+{
+    unsigned long long sum = 0;
+    for (long i = (long)blockIdx.x * blockDim.x + threadIdx.x; i < n_dwords; i += (long)gridDim.x * blockDim.x)
+        sum += (unsigned long long)vals[i] * (2ull * (unsigned long long)i + 1ull);
+#pragma unroll
+    for (int d = 32; d >= 1; d >>= 1) sum += __shfl_xor(sum, d);
+    if ((threadIdx.x & 63) == 0) atomicAdd(out, sum);
+}
+
 // One thread per block: its nonzero columns go to positions padded_start[br] + (offset[p] -
 // offset[row_ptr[br]]) .. of the padded list.
 __global__ void gather_kernel(const uint16_t *__restrict__ vals, const uint16_t *__restrict__ mask,
@@ -353,6 +365,27 @@ hipError_t launch_compact(const CompactArgs &a_in, hipStream_t st)
     return e;
 }
 
+hipError_t values_checksum(const uint16_t *vals, size_t nnzb, uint64_t *out)
+{
+    *out = 0;
+    if (!nnzb) return hipSuccess;
+    unsigned long long *d = nullptr;
+    hipError_t e = hipMalloc(&d, sizeof(unsigned long long));
+    if (e != hipSuccess) return e;
+    e = hipMemset(d, 0, sizeof(unsigned long long));
+    if (e == hipSuccess) {
+        const long n_dwords = (long)nnzb * 128;
+        const unsigned blocks = (unsigned)std::min<long>((n_dwords + 255) / 256, 256L * 16);
+        hipLaunchKernelGGL(values_checksum_kernel, dim3(blocks), dim3(256), 0, 0, reinterpret_cast<const uint32_t *>(vals), n_dwords, d);
+        e = hipGetLastError();
+    }
+    unsigned long long h = 0;
+    if (e == hipSuccess) e = hipMemcpy(&h, d, sizeof h, hipMemcpyDeviceToHost);
+    (void)hipFree(d);
+    *out = h;
+    return e;
+}
+
 void compact_destroy(CompactPlan *p)
 {
     if (!p) return;
@@ -474,6 +507,7 @@ hipError_t compact_build(const uint16_t *vals, const int32_t *row_ptr, const int
         SMAT_STEP(hipMemcpy(p->d_split, split.data(), split.size() * sizeof(SplitRow), hipMemcpyHostToDevice));
         SMAT_STEP(hipMalloc(&p->d_workspace, (size_t)slot * 16 * n_cap * sizeof(float)));
     }
+    SMAT_STEP(values_checksum(vals, nnzb, &p->values_checksum));
     SMAT_STEP(hipDeviceSynchronize());
 #undef SMAT_STEP
     if (e != hipSuccess) {

@@ -75,6 +75,7 @@ struct CompactPlan {
     int n_items = 0, n_split_rows = 0, n_slots = 0;
     int64_t n_cols = 0;           // nonzero block columns listed (without padding)
     int64_t n_cols_all = 0;       // nonzero block columns of the whole matrix
+    uint64_t values_checksum = 0; // of the block values the lists were made from
 };
 // vals / row_ptr / col_idx: device BCSR arrays; row_ptr_host: host copy of row_ptr.
 // dense_rows != NULL and dense_share > 0: block rows with at least that share of nonzero columns get no list and no
@@ -83,6 +84,8 @@ hipError_t compact_build(const uint16_t *vals, const int32_t *row_ptr, const int
                          const int32_t *row_ptr_host, size_t mb, size_t nnzb, size_t n_cap, double dense_share,
                          std::vector<uint8_t> *dense_rows, CompactPlan **out);
 void compact_destroy(CompactPlan *p);
+// Order-independent checksum of nnzb * 256 block values on the device (synchronous, one pass over vals).
+hipError_t values_checksum(const uint16_t *vals, size_t nnzb, uint64_t *out);
 struct CompactArgs {
     const uint16_t *B; // column-major, or row-major with b_row_major
     bool b_row_major;  // B is already B[k*N + n]: no copy is made

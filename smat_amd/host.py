@@ -224,6 +224,12 @@ class Plan:
         ci = None if col_idx_host is None else np.ascontiguousarray(col_idx_host, dtype=np.int32)
         check(lib.smat_plan_check(self._h, _p(rp), _p(ci), M, K, nnzb))
 
+    def values_current(self, vals_dev):
+        """False when the block values have changed since attach_values (the compact kernel works from a copy)."""
+        cur = C.c_int()
+        check(lib.smat_plan_values_current(self._h, C.c_void_p(vals_dev.data_ptr()), C.byref(cur)))
+        return bool(cur.value)
+
     def attach_values(self, vals_dev, row_ptr_dev, col_idx_dev):
         """Let the plan list the nonzero columns of the blocks (device tensors of the same matrix)."""
         ptr = lambda t: C.c_void_p(t.data_ptr()) if t is not None else None  # noqa: E731

@@ -567,3 +567,41 @@ def test_mixed_dispatch_falls_back_to_one_kernel(smat, cuda, oracle):
     assert oracle.compare(C, oracle_ref(oracle, A, B, 64))[0] <= TOL_F16
     with pytest.raises(smat.SmatError, match="SMAT_KERNEL_MIXED needs a plan"):
         gpu_spmm(smat, cuda, A, B, 64, plan=True, kernel=MIXED)
+
+
+def test_values_checksum_tells_when_to_attach_again(smat, cuda, oracle):
+    """The compact kernel multiplies the copy taken by attach_values: after an in-place update of the values the
+    guard says so, the stale result is the old product, and attaching again gives the new one."""
+    import torch
+    d = gen.erdos_renyi(512, 0.01, seed=13)
+    A = bcsr_of(smat, d)
+    M, K, nnzb, N = A["M"], A["K"], A["nnzb"], 64
+    B = gen.dense_b(K, N, seed=14, dist="uniform")
+    vals, rp, ci = to_dev(torch, A["b_val"], cuda), to_dev(torch, A["b_row_ptr"].astype(np.int32), cuda), to_dev(torch, A["b_col_idx"].astype(np.int32), cuda)
+    Bd = to_dev(torch, B, cuda)
+    p = smat.Plan(A["b_row_ptr"], M, K, nnzb, N, col_idx_host=A["b_col_idx"], kernel=COMPACT)
+    p.attach_values(vals, rp, ci)
+    assert p.values_current(vals)
+    new_val = (A["b_val"].view(np.float16) * np.float16(2)).view(np.uint16)
+    vals.copy_(to_dev(torch, new_val, cuda))
+    torch.cuda.synchronize()
+    assert not p.values_current(vals)
+    p.attach_values(vals, rp, ci)
+    assert p.values_current(vals)
+    C = torch.full((M, N), 0x7E00, dtype=torch.int16, device=cuda)
+    smat.spmm(vals, rp, ci, Bd, C, M, N, K, nnzb, plan=p, kernel=COMPACT)
+    torch.cuda.synchronize()
+    A2 = dict(A, b_val=new_val)
+    assert oracle.compare(C.cpu().numpy().view(np.uint16), oracle_ref(oracle, A2, B, N))[0] <= TOL_F16
+    # two values swapped inside one block: same multiset, another checksum
+    v = new_val.copy()
+    nz = np.flatnonzero(v)
+    v[nz[0]], v[nz[-1]] = v[nz[-1]], v[nz[0]]
+    if not np.array_equal(v, new_val):
+        vals.copy_(to_dev(torch, v, cuda))
+        torch.cuda.synchronize()
+        assert not p.values_current(vals)
+    p.close()
+    plain = smat.Plan(A["b_row_ptr"], M, K, nnzb, N, kernel=1)  # no copy of the values: always current
+    assert plain.values_current(vals)
+    plain.close()
