@@ -296,7 +296,7 @@ int smat_event_synchronize(void *event);
 int smat_event_elapsed_ms(void *start, void *stop, float *ms);
 
 /* Benchmark helper (no counterpart in the reference): the fp16 MFMA rate this device reaches on a kernel of
- * nothing but v_mfma_f32_16x16x32_f16 on registers, in TFLOP/s (best of three timed passes, about 1 ms each).
+ * nothing but v_mfma_f32_16x16x32_f16 on registers, in TFLOP/s (best of seven timed passes, about 1 ms each).
  * The published peak assumes the maximum clock; this is what the card sustains. */
 int smat_bench_mfma_peak(double *tflops);
 

@@ -698,9 +698,11 @@ __global__ __launch_bounds__(512) void mfma_peak_kernel(float *out, int iters)
     for (int t = 0; t < 8; t++) acc[t] = (peak_f32x4){0, 0, 0, 0};
     const _Float16 x = (_Float16)(0.001f * (threadIdx.x & 7)), y = (_Float16)(threadIdx.x & 3);
     peak_f16x8 a = {x, x, x, x, x, x, x, x}, b = {y, y, y, y, y, y, y, y};
-    for (int i = 0; i < iters; i++) {
+    for (int i = 0; i < iters; i += 8) { // 64 MFMAs per trip: the loop control disappears behind them
 #pragma unroll
-        for (int t = 0; t < 8; t++) acc[t] = __builtin_amdgcn_mfma_f32_16x16x32_f16(a, b, acc[t], 0, 0, 0);
+        for (int u = 0; u < 8; u++)
+#pragma unroll
+            for (int t = 0; t < 8; t++) acc[t] = __builtin_amdgcn_mfma_f32_16x16x32_f16(a, b, acc[t], 0, 0, 0);
     }
     float s = 0;
     for (int t = 0; t < 8; t++) s += acc[t][0] + acc[t][1] + acc[t][2] + acc[t][3];
@@ -722,7 +724,7 @@ extern "C" int smat_bench_mfma_peak(double *tflops)
     SMAT_HIP(hipEventCreate(&e0));
     SMAT_HIP(hipEventCreate(&e1));
     double best = 0;
-    for (int rep = 0; rep < 4; rep++) { // first pass warms the clocks
+    for (int rep = 0; rep < 8; rep++) { // the first passes warm the clocks
         SMAT_HIP(hipEventRecord(e0, nullptr));
         hipLaunchKernelGGL(mfma_peak_kernel, dim3(cus), dim3(512), 0, nullptr, out, iters);
         SMAT_HIP(hipEventRecord(e1, nullptr));
