@@ -32,9 +32,9 @@ void build_sweep_plan(const int32_t *row_ptr, const int32_t *col_idx, size_t mb,
     out.op_ptr.reserve(n_rg * WAVES + 1);
     out.row_map.assign(n_rg * G, -1);
     std::vector<int32_t> local(n_kchunks, -1); // K chunk -> position in the row group's chunk list
-    struct RowOp { int32_t exec; SweepOpHost op; };
+    struct RowOp { int32_t exec, first, last, hi; SweepOpHost op; }; // nominal chunk period, the periods it may run in, its later chunk
     std::vector<RowOp> row_ops[G];
-    struct Ranked { int rank; int row; SweepOpHost op; };
+    struct Ranked { int rank; int row; int32_t hi; SweepOpHost op; };
     std::vector<std::vector<Ranked>> by_chunk;
     std::vector<int32_t> count; // ops of (row, chunk)
     for (size_t rg = 0; rg < n_rg; rg++) {
@@ -64,15 +64,15 @@ void build_sweep_plan(const int32_t *row_ptr, const int32_t *col_idx, size_t mb,
                 const int32_t cl0 = local[(size_t)bc0 / S];
                 const uint32_t off0 = sweep_lds_offset(cl0, bc0 % S);
                 SweepOpHost op{0, off0, 0, 0};
-                int32_t exec = cl0;
+                int32_t cl_hi = cl0;
                 bool pair = false;
                 if (q + 1 < q_end) {
                     const int32_t bc1 = col_idx[q + 1] / 16;
                     const int32_t cl1 = local[(size_t)bc1 / S];
-                    if (cl1 - cl0 <= 1) { // same chunk or the next listed one: both stages are resident
+                    if (cl1 - cl0 <= 1) { // same chunk or the next listed one (a pair two chunks apart could run in one period only)
                         op.w0 = (uint32_t)q * 512u;
                         op.w2 = sweep_lds_offset(cl1, bc1 % S) - off0;
-                        exec = cl1;
+                        cl_hi = cl1;
                         pair = true;
                     }
                 }
@@ -86,8 +86,12 @@ void build_sweep_plan(const int32_t *row_ptr, const int32_t *col_idx, size_t mb,
                         op.w2 = off0 - SWEEP_ZERO_OFF;
                     }
                 }
+                // While chunk p is swept, chunks p - 1, p and p + 1 are in LDS: the op may run in any period p with
+                // p - 1 <= cl0 and cl_hi <= p + 1.
+                const int32_t first = std::max(cl_hi - 1, 0), last = std::min<int32_t>(cl0 + 1, (int32_t)n_chunks - 1);
+                const int32_t exec = std::min(std::max(cl_hi, first), last);
                 (pair ? out.n_pairs : out.n_singles)++;
-                row_ops[lr].push_back(RowOp{exec, op});
+                row_ops[lr].push_back(RowOp{exec, first, last, cl_hi, op});
                 count[(size_t)lr * n_chunks + (size_t)exec]++;
                 q += pair ? 2 : 1;
             }
@@ -138,24 +142,82 @@ void build_sweep_plan(const int32_t *row_ptr, const int32_t *col_idx, size_t mb,
             }
         }
 
+        // ---- which period every op runs in.  All wavefronts meet at a barrier once per period, so a period costs
+        // the op count of its busiest wavefront.  An op may run one period before or after its nominal one where
+        // its chunks are resident: every period gets a common cap (what has to run now on the busiest wavefront,
+        // or an even share of what is left), and every wavefront runs its pending ops up to the cap, earliest
+        // deadline first. ----
+        struct Pending { int32_t last, first, seq, row, hi, exec; SweepOpHost op; };
+        std::vector<std::vector<std::vector<Ranked>>> schedule((size_t)WAVES, std::vector<std::vector<Ranked>>(n_chunks));
+        if (n_chunks > 0) {
+            std::vector<Pending> todo[WAVES];
+            size_t next[WAVES] = {0}, left = 0;
+            for (int w = 0; w < WAVES; w++) {
+                int r = 0;
+                for (int lr = 0; lr < G; lr++) {
+                    if (wave_of[lr] != w) continue;
+                    if (r_begin + (size_t)lr < r_end) out.row_map[(rg * WAVES + (size_t)w) * RW + (size_t)r] = (int32_t)row_at(r_begin + (size_t)lr);
+                    for (const RowOp &ro : row_ops[lr]) todo[w].push_back(Pending{ro.last, ro.first, (int32_t)todo[w].size(), r, ro.hi, ro.exec, ro.op});
+                    r++;
+                }
+                std::stable_sort(todo[w].begin(), todo[w].end(), [](const Pending &a, const Pending &b) { return a.first < b.first; });
+                left += todo[w].size();
+            }
+            std::vector<Pending> ready[WAVES];
+            size_t left_w[WAVES];
+            for (int w = 0; w < WAVES; w++) left_w[w] = todo[w].size();
+            for (size_t c = 0; c < n_chunks; c++) {
+                // Per wavefront: ops whose nominal period has come (deadline order: what has to run now first), then
+                // those of the next period, which may run early.  The period costs what its busiest wavefront has to
+                // run (its musts, or its own even pace over the periods that are left); every other wavefront uses
+                // that time too, with ops of the next period if it has no others, so that they are gone before
+                // they become musts.  One op of the next period always stays: the first op of a period must not be
+                // an early one.
+                size_t due[WAVES], must[WAVES], cap = MIN_OPS;
+                for (int w = 0; w < WAVES; w++) {
+                    while (next[w] < todo[w].size() && todo[w][next[w]].first <= (int32_t)c) ready[w].push_back(todo[w][next[w]++]);
+                    std::stable_sort(ready[w].begin(), ready[w].end(), [](const Pending &a, const Pending &b) {
+                        if (a.last != b.last) return a.last < b.last;
+                        return a.seq < b.seq;
+                    });
+                    std::stable_partition(ready[w].begin(), ready[w].end(), [&](const Pending &a) { return a.exec <= (int32_t)c; });
+                    due[w] = must[w] = 0;
+                    while (due[w] < ready[w].size() && ready[w][due[w]].exec <= (int32_t)c) due[w]++;
+                    while (must[w] < due[w] && ready[w][must[w]].last <= (int32_t)c) must[w]++;
+                    const size_t pace = (left_w[w] + (n_chunks - c) - 1) / (n_chunks - c);
+                    cap = std::max(cap, std::max(must[w], std::min(due[w], pace)));
+                }
+                for (int w = 0; w < WAVES; w++) {
+                    const size_t early = ready[w].size() - due[w];
+                    size_t k = std::max(must[w], std::min(due[w], cap));
+                    size_t pull = 0;
+                    if (k < cap && early > 1) pull = std::min(early - 1, cap - k);
+                    if (pull) { // the early ops to run sit behind the due ones that wait: bring them forward
+                        std::rotate(ready[w].begin() + (long)k, ready[w].begin() + (long)due[w], ready[w].begin() + (long)(due[w] + pull));
+                        k += pull;
+                    }
+                    std::vector<Ranked> &list = schedule[(size_t)w][c];
+                    for (size_t x = 0; x < k; x++) {
+                        const Pending &pe = ready[w][x];
+                        // rank = how many ops of this block row the period already holds: ops of one block
+                        // row (same accumulators) end up spread over the period
+                        int rank = 0;
+                        for (const Ranked &y : list) rank += y.row == pe.row;
+                        list.push_back(Ranked{rank, pe.row, pe.hi, pe.op});
+                    }
+                    ready[w].erase(ready[w].begin(), ready[w].begin() + (long)k);
+                    left_w[w] -= k;
+                    left -= k;
+                }
+            }
+            if (left) throw std::logic_error("sweep plan: ops left over by the period schedule");
+        }
+
         // ---- streams: ops of chunk 0, marker, ops of chunk 1, ..., end ----
         for (int w = 0; w < WAVES; w++) {
             out.op_ptr.push_back((int32_t)out.ops.size());
             if (n_chunks == 0) continue; // the kernel does not enter the interpreter for an empty row group
-            by_chunk.assign(n_chunks, {});
-            int r = 0;
-            for (int lr = 0; lr < G; lr++) {
-                if (wave_of[lr] != w) continue;
-                if (r_begin + (size_t)lr < r_end) out.row_map[(rg * WAVES + (size_t)w) * RW + (size_t)r] = (int32_t)row_at(r_begin + (size_t)lr);
-                for (const RowOp &ro : row_ops[lr]) {
-                    // rank = how many ops of this block row the chunk already holds: ops of one block
-                    // row (same accumulators) end up spread over the chunk
-                    int rank = 0;
-                    for (const Ranked &x : by_chunk[(size_t)ro.exec]) rank += x.row == r;
-                    by_chunk[(size_t)ro.exec].push_back(Ranked{rank, r, ro.op});
-                }
-                r++;
-            }
+            by_chunk = schedule[(size_t)w];
             struct Item { int kind, row; SweepOpHost op; }; // kind: 0 op, 1 marker, 2 end
             std::vector<Item> items;
             const SweepOpHost idle{0, SWEEP_ZERO_OFF, 0, 0}; // blocks 0 and 1 times zeros
@@ -165,7 +227,19 @@ void build_sweep_plan(const int32_t *row_ptr, const int32_t *col_idx, size_t mb,
                     if (a.rank != b.rank) return a.rank < b.rank;
                     return a.row < b.row;
                 });
-                if (c > 0) items.push_back(Item{1, 0, idle});
+                if (c > 0) {
+                    items.push_back(Item{1, 0, idle});
+                    // The LDS reads of the first op after a marker are issued before the marker's barrier, when the
+                    // copies of chunk c + 1 may still be under way: that op has to be one whose chunks are c or c - 1.
+                    size_t ok = 0;
+                    while (ok < list.size() && list[ok].hi > (int32_t)c) ok++;
+                    if (ok == list.size()) {
+                        items.push_back(Item{0, 0, idle});
+                        out.n_fillers++;
+                    } else if (ok > 0) {
+                        std::rotate(list.begin(), list.begin() + (long)ok, list.begin() + (long)ok + 1);
+                    }
+                }
                 for (const Ranked &x : list) items.push_back(Item{0, x.row, x.op});
                 for (size_t k = list.size(); k < (size_t)MIN_OPS; k++) { // filler ops keep the markers AHEAD positions apart
                     items.push_back(Item{0, 0, idle});
