@@ -69,7 +69,7 @@ void build_sweep_plan(const int32_t *row_ptr, const int32_t *col_idx, size_t mb,
                 if (q + 1 < q_end) {
                     const int32_t bc1 = col_idx[q + 1] / 16;
                     const int32_t cl1 = local[(size_t)bc1 / S];
-                    if (cl1 - cl0 <= 1) { // same chunk or the next listed one (a pair two chunks apart could run in one period only)
+                    if (cl1 - cl0 <= 2) { // three consecutive listed chunks are resident while the middle one is swept
                         op.w0 = (uint32_t)q * 512u;
                         op.w2 = sweep_lds_offset(cl1, bc1 % S) - off0;
                         cl_hi = cl1;
