@@ -57,7 +57,8 @@ struct smat_plan {
     bool fingerprint_has_cols = false;
     // compacted-column kernel (present after smat_plan_attach_values)
     CompactPlan *compact = nullptr;
-    uint16_t *d_bt = nullptr; // row-major copy of B, K * n_cap halves (compact kernel)
+    uint16_t *d_bt = nullptr; // copy of B in panels of rows, K * (n_cap rounded up to 256) halves (compact kernel)
+    size_t bt_bytes() const { return K * ((n_cap + 255) / 256 * 256) * sizeof(uint16_t); }
     // mixed dispatch (after smat_plan_attach_values): row-wise work list of the block rows with mostly full blocks
     WorkItem *d_items_dense = nullptr;
     SplitRow *d_split_dense = nullptr;
@@ -509,7 +510,7 @@ static int smat_plan_attach_values_impl(smat_plan *p, const uint16_t *vals, cons
         if (p->kernel == SMAT_KERNEL_COMPACT || p->kernel == SMAT_KERNEL_MIXED) p->kernel = dense_kernel;
         return SMAT_OK;
     }
-    if (!p->d_bt) e = hipMalloc(&p->d_bt, p->K * p->n_cap * sizeof(uint16_t));
+    if (!p->d_bt) e = hipMalloc(&p->d_bt, p->bt_bytes());
     // the dense rows through the sweep kernel when their row groups of 64 fill the device, else row-wise
     std::vector<int32_t> dense_list;
     for (size_t i = 0; mixed && i < mb; i++)
@@ -610,7 +611,7 @@ extern "C" int smat_plan_info(const smat_plan *p, int64_t *info)
     info[5] = p->kernel == SMAT_KERNEL_SWEEP ? 16 * SWEEP_TN : 16 * p->panel_tiles;
     info[6] = p->sweep.n_ops + p->sweep_dense.n_ops; info[7] = p->sweep.n_records + p->sweep_dense.n_records;
     info[8] = (p->d_bpack ? (int64_t)(p->K * p->n_cap * sizeof(uint16_t)) : 0) +
-              (p->d_bt ? (int64_t)(p->K * p->n_cap * sizeof(uint16_t)) : 0) +
+              (p->d_bt ? (int64_t)p->bt_bytes() : 0) +
               (p->d_bcol ? (int64_t)(p->K * p->n_cap * sizeof(uint16_t)) : 0);
     info[9] = p->compact ? p->compact->n_cols : 0;
     info[10] = p->n_items_dense; info[11] = p->n_blocks_dense;

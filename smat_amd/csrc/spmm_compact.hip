@@ -19,8 +19,10 @@
 //                       so that the A operand of a step is one coalesced 16-byte load per lane.
 //    The SpMM then does not read the block values any more: they must be attached again when
 //    they change.
-//  * transpose_b_kernel: column-major B (B[n*K + k]) -> row-major Bt[k*N + n] at the start of
-//    every launch, so that the row of B under a nonzero column is contiguous.
+//  * transpose_b_kernel: column-major B (B[n*K + k]) -> Bt at the start of every launch, so that
+//    the row of B under a nonzero column is contiguous.  Bt holds the panels of 64*TQ columns one
+//    after the other, each a row-major K x 64*TQ matrix: the pass over a panel gathers from one
+//    contiguous K * 128*TQ bytes.
 //  * spmm_compact_kernel<TQ>: one wavefront per (work item, panel of 64*TQ columns).  A step takes
 //    32 columns = K of one v_mfma_f32_16x16x32_f16.  The product is formed as
 //    C^T = B^T * A^T like in the other kernels:
@@ -143,8 +145,10 @@ __global__ void row_offsets_kernel(const int32_t *__restrict__ row_ptr, const in
 // 64 n x 64 k tile through LDS.  A thread reads 16 bytes (8 k) of two neighbouring columns, pairs
 // the values of equal k into dwords and writes them to the transposed tile; then every thread
 // reads 8 n of one k back (two 8-byte LDS reads) and stores 16 bytes.
+// The output is split into panels of `panel` columns, each a K x panel row-major matrix of leading
+// dimension ld, one panel after the other (panel >= N and ld = N: plain row-major K x N).
 __global__ __launch_bounds__(256) void transpose_b_kernel(const uint16_t *__restrict__ B, uint16_t *__restrict__ Bt,
-                                                          int N, long K)
+                                                          int N, long K, int panel, long ld)
 {
     constexpr int LD = 68; // halfs per LDS row (k): 8-byte aligned rows, dword writes spread over the banks
     __shared__ __align__(16) uint16_t tile[64 * LD];
@@ -173,18 +177,22 @@ __global__ __launch_bounds__(256) void transpose_b_kernel(const uint16_t *__rest
         if (k0 + k < K && n0 + seg * 8 < N) {
             const uint2 lo = *reinterpret_cast<const uint2 *>(tile + k * LD + seg * 8);
             const uint2 hi = *reinterpret_cast<const uint2 *>(tile + k * LD + seg * 8 + 4);
-            *reinterpret_cast<u32x4 *>(Bt + (k0 + k) * (long)N + n0 + seg * 8) = (u32x4){lo.x, lo.y, hi.x, hi.y};
+            uint16_t *out = Bt + (long)(n0 / panel) * K * panel + (k0 + k) * ld + n0 % panel + seg * 8;
+            *reinterpret_cast<u32x4 *>(out) = (u32x4){lo.x, lo.y, hi.x, hi.y};
         }
     }
 }
 
 // ---- the product ----
 
+#ifndef COMPACT_KERNEL_ATTR
+#define COMPACT_KERNEL_ATTR
+#endif
 template <int TQ, bool C_F32>
-__global__ __launch_bounds__(256) void spmm_compact_kernel(
+__global__ __launch_bounds__(256) COMPACT_KERNEL_ATTR void spmm_compact_kernel(
     const uint16_t *__restrict__ acol, const int32_t *__restrict__ cols, const uint16_t *__restrict__ Bt,
     void *__restrict__ Cout, float *__restrict__ workspace, const WorkItem *__restrict__ items, int n_items, int N,
-    int n_panels)
+    int n_panels, long panel_stride, long row_stride)
 {
     constexpr int PANEL = 64 * TQ;
     const int lane = threadIdx.x & 63;
@@ -195,8 +203,13 @@ __global__ __launch_bounds__(256) void spmm_compact_kernel(
     const long wg = (long)(blockIdx.x & 7) * chunk + (blockIdx.x >> 3);
     const long w = wg * 4 + wave;
     if (w >= total) return;
+#ifdef COMPACT_ITEM_MAJOR
+    const int it = (int)(w / n_panels);
+    const int panel = (int)(w - (long)it * n_panels);
+#else
     const int panel = (int)(w / n_items);
     const int it = (int)(w - (long)panel * n_items);
+#endif
     const WorkItem wi = items[it];
     const int br = __builtin_amdgcn_readfirstlane(wi.block_row);
     const int e0 = __builtin_amdgcn_readfirstlane(wi.begin);
@@ -205,11 +218,14 @@ __global__ __launch_bounds__(256) void spmm_compact_kernel(
 
     const int i16 = lane & 15, g = lane >> 4;
     const int n0 = panel * PANEL;
-    long boff[TQ]; // element offset of this lane's 4 columns inside a row of Bt (column 0 when out of range)
+    // Row `col` of this panel of B starts at Bp + col * row_stride (B in place: panel_stride = PANEL,
+    // row_stride = N; the transposed copy: panels one after the other, row_stride = PANEL).
+    const uint16_t *Bp = Bt + (long)panel * panel_stride;
+    int boff[TQ]; // element offset of this lane's 4 columns inside the panel row (its column 0 when out of range)
 #pragma unroll
     for (int q = 0; q < TQ; q++) {
-        const int n = n0 + 64 * q + 4 * i16;
-        boff[q] = n < N ? n : 0; // N % 8 == 0: all four columns or none
+        const int n = 64 * q + 4 * i16;
+        boff[q] = n0 + n < N ? n : 0; // N % 8 == 0: all four columns or none
     }
 
     f32x4 acc[TQ][4];
@@ -235,7 +251,7 @@ __global__ __launch_bounds__(256) void spmm_compact_kernel(
         for (int q = 0; q < TQ; q++)
 #pragma unroll
             for (int j = 0; j < 8; j++)
-                o.L[q][j] = *reinterpret_cast<const uint2 *>(Bt + (long)col[j] * N + boff[q]);
+                o.L[q][j] = *reinterpret_cast<const uint2 *>(Bp + (long)col[j] * row_stride + boff[q]);
     };
     auto multiply = [&](const Operands &o) {
         const f16x8 av = __builtin_bit_cast(f16x8, o.aw);
@@ -310,7 +326,17 @@ template <int TQ>
 hipError_t launch_compact_tq(const CompactArgs &a, hipStream_t st)
 {
     const CompactPlan &p = *a.plan;
-    const int n_panels = (int)((a.N + 64 * TQ - 1) / (64 * TQ));
+    constexpr int PANEL = 64 * TQ;
+    const int n_panels = (int)((a.N + PANEL - 1) / PANEL);
+    long panel_stride = PANEL, row_stride = (long)a.N;
+    if (!a.b_row_major) {
+        dim3 grid((unsigned)((a.K + 63) / 64), (unsigned)((a.N + 63) / 64));
+        hipLaunchKernelGGL(transpose_b_kernel, grid, dim3(256), 0, st, a.B, a.Bt, (int)a.N, (long)a.K, PANEL, (long)PANEL);
+        hipError_t e = hipGetLastError();
+        if (e != hipSuccess) return e;
+        panel_stride = (long)a.K * PANEL;
+        row_stride = PANEL;
+    }
     const long total = (long)p.n_items * n_panels;
     long wgs = (total + 3) / 4;
     wgs = (wgs + 7) / 8 * 8;
@@ -318,10 +344,10 @@ hipError_t launch_compact_tq(const CompactArgs &a, hipStream_t st)
     if (wgs > 0x7fffffffL) return hipErrorInvalidValue;
     if (a.c_f32)
         hipLaunchKernelGGL((spmm_compact_kernel<TQ, true>), dim3((unsigned)wgs), dim3(256), 0, st, p.d_acol, p.d_cols,
-                           a.Bt, a.C, p.d_workspace, p.d_items, p.n_items, (int)a.N, n_panels);
+                           a.Bt, a.C, p.d_workspace, p.d_items, p.n_items, (int)a.N, n_panels, panel_stride, row_stride);
     else
         hipLaunchKernelGGL((spmm_compact_kernel<TQ, false>), dim3((unsigned)wgs), dim3(256), 0, st, p.d_acol, p.d_cols,
-                           a.Bt, a.C, p.d_workspace, p.d_items, p.n_items, (int)a.N, n_panels);
+                           a.Bt, a.C, p.d_workspace, p.d_items, p.n_items, (int)a.N, n_panels, panel_stride, row_stride);
     return hipGetLastError();
 }
 
@@ -338,7 +364,7 @@ struct Scratch {
 hipError_t launch_b_to_col_major(const uint16_t *B_row_major, uint16_t *out, size_t N, size_t K, hipStream_t st)
 {
     dim3 grid((unsigned)((N + 63) / 64), (unsigned)((K + 63) / 64));
-    hipLaunchKernelGGL(transpose_b_kernel, grid, dim3(256), 0, st, B_row_major, out, (int)K, (long)N);
+    hipLaunchKernelGGL(transpose_b_kernel, grid, dim3(256), 0, st, B_row_major, out, (int)K, (long)N, 0x7fffffff, (long)K);
     return hipGetLastError();
 }
 
@@ -346,18 +372,23 @@ hipError_t launch_compact(const CompactArgs &a_in, hipStream_t st)
 {
     CompactArgs a = a_in;
     hipError_t e = hipSuccess;
-    if (a.b_row_major) {
-        a.Bt = const_cast<uint16_t *>(a.B); // read in place, never written
-    } else {
-        dim3 grid((unsigned)((a.K + 63) / 64), (unsigned)((a.N + 63) / 64));
-        hipLaunchKernelGGL(transpose_b_kernel, grid, dim3(256), 0, st, a.B, a.Bt, (int)a.N, (long)a.K);
-        e = hipGetLastError();
-        if (e != hipSuccess) return e;
-    }
-    // wide panels reuse the A operand over more columns; narrow ones give more wavefronts
+    if (a.b_row_major) a.Bt = const_cast<uint16_t *>(a.B); // read in place, never written
+    // Wide panels reuse the A operand over more columns; narrow ones give more wavefronts.  The
+    // panels are swept one after the other, so the rows of B that the gathers hit at random come
+    // from one panel at a time: a panel is kept under half of the 256 MiB memory-side cache (the
+    // lists of A and the rows of C stream through it too).  On a 2^20-row B at N = 128 the panel
+    // of 64 columns (128 MiB) takes 0.74 x the time of the panel of 128.
     const long items = a.plan->n_items;
-    if (a.N >= 256 && items * (long)(a.N / 256) >= 4096) e = launch_compact_tq<4>(a, st);
-    else if (a.N >= 128 && items * (long)(a.N / 128) >= 2048) e = launch_compact_tq<2>(a, st);
+    int tq = 1;
+    if (a.N >= 256 && items * (long)(a.N / 256) >= 4096) tq = 4;
+    else if (a.N >= 128 && items * (long)(a.N / 128) >= 2048) tq = 2;
+#ifdef COMPACT_FORCE_TQ
+    tq = COMPACT_FORCE_TQ;
+#else
+    while (tq > 1 && a.K * (size_t)(64 * tq) * sizeof(uint16_t) > ((size_t)128 << 20)) tq >>= 1;
+#endif
+    if (tq == 4) e = launch_compact_tq<4>(a, st);
+    else if (tq == 2) e = launch_compact_tq<2>(a, st);
     else e = launch_compact_tq<1>(a, st);
     if (e != hipSuccess) return e;
     if (a.plan->n_split_rows > 0)

@@ -89,7 +89,7 @@ hipError_t values_checksum(const uint16_t *vals, size_t nnzb, uint64_t *out);
 struct CompactArgs {
     const uint16_t *B; // column-major, or row-major with b_row_major
     bool b_row_major;  // B is already B[k*N + n]: no copy is made
-    uint16_t *Bt;      // scratch, K * N halves: row-major copy of B made at the start of the launch
+    uint16_t *Bt;      // scratch, K * (N rounded up to 256) halves: the copy of B in panels of rows made at the start of the launch
     void *C;
     size_t M, N, K;
     bool c_f32;
