@@ -38,7 +38,10 @@
 #include <cstdint>
 #include <cstdlib>
 #include <cstring>
+#include <atomic>
+#include <functional>
 #include <numeric>
+#include <thread>
 #include <utility>
 #include <vector>
 
@@ -52,16 +55,19 @@ namespace {
 // _Rb_tree (insert_and_rebalance / rebalance_for_erase).  Index 0 is "null".
 class CandidateTree {
 public:
-    struct Node {
+    struct Node { // 24 bytes: the set grows to tens of thousands of rows on power-law matrices
         float dist;
-        int64_t row;
+        int32_t row;
         int32_t parent, left, right;
-        bool red;
+        bool red, alive;
     };
 
     void clear()
     {
         nodes_.resize(1);
+        free_.clear();
+        generation_++; // forgets every hint
+        hints_used_ = 0;
         root_ = 0;
         rightmost_ = 0;
         leftmost_ = 0;
@@ -69,17 +75,46 @@ public:
     }
     size_t size() const { return size_; }
 
+    // Rows come in ascending order, and the distances take few different values (they are ratios of small
+    // block counts): the node that was inserted last with the same distance, if it is still in the tree, is the
+    // in-order predecessor of the new key, and a key goes below its predecessor (if that has no right child) or
+    // below its successor (the leftmost node of that right subtree).  With unique keys a search tree has one
+    // place for a key, so this is the place the descent from the root ends at, found without the descent.
     void insert(float dist, int64_t row)
     {
-        int32_t y = 0, x = root_;
+        int32_t y = 0;
         bool less_than = true;
-        while (x) {
-            y = x;
-            less_than = key_less(dist, row, nodes_[x]);
-            x = less_than ? nodes_[x].left : nodes_[x].right;
+        Hint *hint = hint_for(dist);
+        const int32_t h = hint && hint->generation == generation_ ? hint->node : 0;
+        if (h && nodes_[h].alive && nodes_[h].dist == dist && nodes_[h].row < row) {
+            if (!nodes_[h].right) {
+                y = h;
+                less_than = false;
+            } else {
+                y = nodes_[h].right;
+                while (nodes_[y].left) y = nodes_[y].left;
+            }
+        } else {
+            int32_t x = root_;
+            while (x) {
+                y = x;
+                less_than = key_less(dist, row, nodes_[x]);
+                x = less_than ? nodes_[x].left : nodes_[x].right;
+            }
         }
-        nodes_.push_back(Node{dist, row, y, 0, 0, true});
-        const int32_t z = (int32_t)nodes_.size() - 1;
+        int32_t z;
+        if (!free_.empty()) { // which slot a node lives in does not show in the shape of the tree
+            z = free_.back();
+            free_.pop_back();
+            nodes_[z] = Node{dist, (int32_t)row, y, 0, 0, true, true};
+        } else {
+            nodes_.push_back(Node{dist, (int32_t)row, y, 0, 0, true, true});
+            z = (int32_t)nodes_.size() - 1;
+        }
+        if (hint) {
+            if (hint->generation != generation_) hints_used_++;
+            *hint = Hint{dist, z, generation_};
+        }
         if (!y) {
             root_ = leftmost_ = rightmost_ = z;
         } else if (less_than) {
@@ -91,6 +126,15 @@ public:
         }
         ++size_;
         insert_fixup(z);
+    }
+
+    // True if insert(dist, row) followed by trim_from_end(steps) with an odd `steps` would leave the tree as it is:
+    // a key above the largest one becomes the right child of the largest node; under a black parent nothing is
+    // rebalanced; the new node, a red leaf without a left child, is then the only one the trim removes (cycle of
+    // two, odd step count), and removing a red leaf rebalances nothing either.
+    bool insert_then_trim_is_noop(float dist, int64_t row) const
+    {
+        return rightmost_ && !nodes_[rightmost_].red && !key_less(dist, row, nodes_[rightmost_]);
     }
 
     // Emulates `it = end(); advance(it, steps); erase(it, end());`.
@@ -280,10 +324,35 @@ private:
             if (x) nodes_[x].red = false;
         }
         --size_;
-        // the erased slot stays in the pool until clear(); it is unreachable
+        nodes_[z].alive = false;
+        free_.push_back(z); // unlinked above (y == z by now): the slot is reused by the next insert
+    }
+
+    // distance -> node inserted last with it: open addressing, entries of an older generation are free
+    struct Hint {
+        float dist;
+        int32_t node;
+        uint32_t generation;
+    };
+    static constexpr size_t HINTS = 4096;
+    Hint *hint_for(float dist)
+    {
+        uint32_t bits;
+        memcpy(&bits, &dist, 4);
+        size_t at = (bits * 2654435761u) >> 20; // 12 bits
+        for (size_t probe = 0; probe < 16; probe++, at = (at + 1) & (HINTS - 1)) {
+            Hint &e = hints_[at];
+            if (e.generation != generation_) return hints_used_ < HINTS / 2 ? &e : nullptr;
+            if (e.dist == dist) return &e;
+        }
+        return nullptr; // crowded: this distance goes without a hint
     }
 
     std::vector<Node> nodes_{1};
+    std::vector<int32_t> free_;
+    std::vector<Hint> hints_ = std::vector<Hint>(HINTS, Hint{0.0f, 0, 0});
+    uint32_t generation_ = 1;
+    size_t hints_used_ = 0;
     int32_t root_ = 0, leftmost_ = 0, rightmost_ = 0;
     size_t size_ = 0;
 };
@@ -322,7 +391,125 @@ std::vector<int64_t> permutation_by_group(const std::vector<int64_t> &grouping)
     return v;
 }
 
+// Helper threads for the row scan of keeper_grouping.  A job is a function of the thread index that every
+// thread (the caller as index 0) runs once; run() returns when all have.  Helpers spin between jobs (jobs
+// follow each other within microseconds) and yield when none comes for a while.
+class ScanPool {
+public:
+    explicit ScanPool(int n_threads) : n_(std::max(n_threads, 1))
+    {
+        for (int t = 1; t < n_; t++) helpers_.emplace_back([this, t] { loop(t); });
+    }
+    ~ScanPool()
+    {
+        stop_.store(true, std::memory_order_release);
+        generation_.fetch_add(1, std::memory_order_release);
+        for (std::thread &h : helpers_) h.join();
+    }
+    int size() const { return n_; }
+    // All threads, the caller included, run the job; returns when every one has.
+    void run(const std::function<void(int)> &job)
+    {
+        if (n_ == 1) { job(0); return; }
+        start(job);
+        job(0);
+        wait();
+    }
+    // The helpers run the job while the caller does something else; wait() before the next start() or run().
+    void start(const std::function<void(int)> &job)
+    {
+        if (n_ == 1) return;
+        job_ = &job;
+        pending_.store(n_ - 1, std::memory_order_relaxed);
+        generation_.fetch_add(1, std::memory_order_release);
+    }
+    void wait()
+    {
+        while (pending_.load(std::memory_order_acquire)) spin_pause();
+    }
+
+private:
+    static void spin_pause()
+    {
+#if defined(__x86_64__) || defined(__i386__)
+        __builtin_ia32_pause();
+#endif
+    }
+    void loop(int t)
+    {
+        uint64_t seen = 0;
+        for (;;) {
+            int idle = 0;
+            while (generation_.load(std::memory_order_acquire) == seen) {
+                if (++idle < 4096) spin_pause();
+                else std::this_thread::yield();
+            }
+            seen = generation_.load(std::memory_order_acquire);
+            if (stop_.load(std::memory_order_acquire)) return;
+            (*job_)(t);
+            pending_.fetch_sub(1, std::memory_order_release);
+        }
+    }
+    const int n_;
+    std::vector<std::thread> helpers_;
+    const std::function<void(int)> *job_ = nullptr;
+    std::atomic<uint64_t> generation_{0};
+    std::atomic<int> pending_{0};
+    std::atomic<bool> stop_{false};
+};
+
+// Threads for the scan: SMAT_REORDER_THREADS, else the hardware's count, at most 16.
+int scan_threads()
+{
+    if (const char *e = getenv("SMAT_REORDER_THREADS")) {
+        const int n = atoi(e);
+        if (n >= 1) return std::min(n, 256);
+    }
+    const unsigned hw = std::thread::hardware_concurrency();
+    return (int)std::min(std::max(hw, 1u), 16u);
+}
+
+// What looking at a row needs, by value: the helper threads take a copy per job, so that they read nothing that
+// the scanning thread writes while it applies results (its locals share cache lines with these fields otherwise).
+struct RowView {
+    static constexpr float PRUNED = -1.0f, TAKEN = -2.0f; // marks next to the distances (which are >= 0)
+    const int64_t *row_ptr, *pat_ptr, *stamp, *grouping;
+    const int32_t *pat_blk;
+    const float *dist_cache;
+    int64_t seed, pattern_blocks, group_size;
+    float seed_cached, tau;
+    bool pattern_empty;
+
+    // what the reference does with row j before it touches any state: skipped by the cached distances,
+    // already in a group, or compared with the pattern
+    float look(int64_t j) const
+    {
+        if (seed_cached != -1 && dist_cache[j] != -1 && std::fabs(seed_cached - dist_cache[j]) > tau) return PRUNED;
+        if (grouping[j] != -1) return TAKEN;
+        const int64_t nb = pat_ptr[j + 1] - pat_ptr[j];
+        const bool b_empty = row_ptr[j + 1] == row_ptr[j];
+        if (pattern_empty && b_empty) return 0.0f;
+        if (pattern_empty || b_empty) return 1.0f;
+        int64_t common = 0;
+        for (int64_t k = pat_ptr[j]; k < pat_ptr[j + 1]; k++) common += stamp[pat_blk[k]] == seed;
+        const int64_t na = pattern_blocks;
+        // count_zeros weighting: blocks only in the group count once, blocks
+        // only in the row count group_size times (blocking.cpp:912-917)
+        const int64_t count = (na - common) + (nb - common) * group_size;
+        return (float)((2.0 * (double)count) / (double)(na * group_size + nb + count));
+    }
+};
+
 // IterativeBlockingKeeper with use_pattern = 1 and the Jaccard group distance.
+//
+// The scan over the later rows j of one seed row i is sequential in the reference: the distance of row j is
+// taken against the pattern as the merges before j left it.  Here the scan runs in batches.  What happens to
+// row j depends on the scan so far only through the pattern and the group size, which change at a merge and
+// nowhere else (at most row_block - 1 times per seed): the rows of a batch are therefore evaluated in
+// parallel against the current pattern, and their results are applied in row order up to and including the
+// first merge; what was evaluated behind it is thrown away and the next batch starts there.  Every write
+// (distance cache, grouping, candidate set, counters) happens in that ordered pass, so the output is the one
+// of the sequential scan whatever the number of threads.
 std::vector<int64_t> keeper_grouping(int64_t rows, const int64_t *row_ptr, const int64_t *col_idx,
                                      const Pattern &pat, int64_t nblk_cols, int64_t col_block,
                                      int64_t max_rows, float tau, int64_t &comparisons,
@@ -337,6 +524,26 @@ std::vector<int64_t> keeper_grouping(int64_t rows, const int64_t *row_ptr, const
     std::vector<int64_t> merged_rows;
     CandidateTree candidates;
 
+    constexpr float TAKEN = RowView::TAKEN;
+    // Row by row for SERIAL_ROWS rows behind a change of the pattern, then batches that grow with the distance
+    // from it.  The two environment variables exist for the tests, which run small matrices through the batches.
+    auto tunable = [](const char *name, int64_t fallback) {
+        const char *e = getenv(name);
+        const long long v = e ? atoll(e) : 0;
+        return v >= 1 ? (int64_t)v : fallback;
+    };
+    const int64_t SERIAL_ROWS = tunable("SMAT_REORDER_SERIAL_ROWS", 512), FIRST_BATCH = tunable("SMAT_REORDER_FIRST_BATCH", 4096);
+    const int64_t MAX_BATCH = std::max<int64_t>(131072, FIRST_BATCH), GRAIN = std::max<int64_t>(1, std::min<int64_t>(512, FIRST_BATCH / 8));
+    const int want_threads = rows >= 4 * FIRST_BATCH ? scan_threads() : 1;
+    ScanPool pool(want_threads);
+    // Three result buffers: one being applied, one being filled for the rows behind it, one whose distances
+    // are being copied into the cache.
+    std::vector<float> results[3];
+    if (pool.size() > 1)
+        for (std::vector<float> &r : results) r.resize((size_t)std::min<int64_t>(rows, MAX_BATCH));
+    struct Span { int buf; int64_t first, count; };
+    std::atomic<int64_t> next_store{0}, next_look{0};
+
     for (int64_t i = 0; i < rows; i++) {
         if (grouping[i] != -1) continue;
         candidates.clear();
@@ -350,71 +557,171 @@ std::vector<int64_t> keeper_grouping(int64_t rows, const int64_t *row_ptr, const
         for (int32_t b : pattern) stamp[b] = i;
         bool pattern_empty = row_ptr[i + 1] == row_ptr[i];
         int64_t pattern_max = pattern_empty ? -1 : col_idx[row_ptr[i + 1] - 1];
+        const float seed_cached = dist_cache[i];
+        auto view = [&] {
+            return RowView{row_ptr, pat.ptr.data(), stamp.data(), grouping.data(), pat.blk.data(), dist_cache.data(),
+                           i, (int64_t)pattern.size(), group_size, seed_cached, tau, pattern_empty};
+        };
 
-        for (int64_t j = i + 1; j < rows; j++) {
-            if (group_size == max_rows) break;
-            if (dist_cache[i] != -1 && dist_cache[j] != -1 &&
-                std::fabs(dist_cache[i] - dist_cache[j]) > tau) {
-                dist_cache[j] = -1;
+        auto look = [&](int64_t j) { return view().look(j); };
+        // a compared row that is not merged competes for the places left in the group
+        auto keep_candidate = [&](int64_t j, float dist) {
+            const size_t room = (size_t)(max_rows - (int64_t)merged_rows.size());
+            // most rows are farther than every candidate kept so far: see insert_then_trim_is_noop
+            if (candidates.size() >= room && (room & 1) && candidates.insert_then_trim_is_noop(dist, j)) return;
+            candidates.insert(dist, j);
+            if (candidates.size() > room) candidates.trim_from_end(room);
+        };
+        auto merge = [&](int64_t j) {
+            merges++;
+            grouping[j] = group_number;
+            merged_rows.push_back(j);
+            // merge_rows(pattern, row j): row j's columns, plus the pattern's
+            // columns below the largest column of row j that is <= max(pattern).
+            // An empty row j therefore empties the pattern.
+            const bool b_empty = row_ptr[j + 1] == row_ptr[j];
+            int64_t cut = -1; // pattern blocks with id < cut survive
+            if (!b_empty && !pattern_empty) {
+                const int64_t *bb = col_idx + row_ptr[j], *be = col_idx + row_ptr[j + 1];
+                const int64_t *ub = std::upper_bound(bb, be, pattern_max);
+                if (ub != bb) cut = *(ub - 1) / col_block;
+            }
+            scratch.clear();
+            for (int32_t b : pattern) {
+                if (b < cut) scratch.push_back(b);
+                else stamp[b] = -1;
+            }
+            pattern.clear();
+            size_t a = 0;
+            int64_t k = pat.ptr[j];
+            while (a < scratch.size() || k < pat.ptr[j + 1]) {
+                if (k >= pat.ptr[j + 1] || (a < scratch.size() && scratch[a] < pat.blk[k])) {
+                    pattern.push_back(scratch[a++]);
+                } else {
+                    if (a < scratch.size() && scratch[a] == pat.blk[k]) a++;
+                    pattern.push_back(pat.blk[k++]);
+                }
+            }
+            for (int32_t b : pattern) stamp[b] = i;
+            pattern_empty = b_empty;
+            pattern_max = b_empty ? -1 : col_idx[row_ptr[j + 1] - 1];
+            group_size++;
+        };
+        // one row, start to end; true if it was merged
+        auto scan_row = [&](int64_t j) -> bool {
+            const float r = look(j);
+            if (r == TAKEN) return false;
+            dist_cache[j] = r; // PRUNED is the cache's own mark for "unknown"
+            if (r < 0) return false;
+            comparisons++;
+            if (r > tau) {
+                keep_candidate(j, r);
+                return false;
+            }
+            merge(j);
+            return true;
+        };
+
+        int64_t j = i + 1;
+        int64_t since_change = 0; // rows scanned since the pattern last changed
+        if (pool.size() == 1) {
+            for (; j < rows && group_size != max_rows; j++) scan_row(j);
+        }
+        // ---- with helpers: `looked` = rows whose results are in a buffer, `stored` = rows applied whose distances
+        // still have to go into the cache (the helpers do that on their next job) ----
+        Span looked{0, 0, 0}, stored{0, 0, 0}, ahead{0, 0, 0};
+        auto free_buffer = [&] { // the one that neither `looked` nor `stored` uses
+            for (int b = 0; b < 3; b++)
+                if (!(looked.count && looked.buf == b) && !(stored.count && stored.buf == b)) return b;
+            return 0; // not reached
+        };
+        // helpers' job: results of `st` into the distance cache, then rows of `lk` looked at
+        Span job_store{0, 0, 0}, job_look{0, 0, 0};
+        RowView job_view = view();
+        const std::function<void(int)> job = [&](int) {
+            const RowView v = job_view;
+            const Span st = job_store, lk = job_look;
+            float *cache = dist_cache.data();
+            for (;;) {
+                const int64_t g0 = next_store.fetch_add(GRAIN, std::memory_order_relaxed);
+                if (g0 >= st.count) break;
+                const int64_t g1 = std::min(st.count, g0 + GRAIN);
+                const float *res = results[st.buf].data();
+                for (int64_t x = g0; x < g1; x++)
+                    if (res[x] != TAKEN) cache[st.first + x] = res[x];
+            }
+            for (;;) {
+                const int64_t g0 = next_look.fetch_add(GRAIN, std::memory_order_relaxed);
+                if (g0 >= lk.count) break;
+                const int64_t g1 = std::min(lk.count, g0 + GRAIN);
+                float *res = results[lk.buf].data();
+                for (int64_t x = g0; x < g1; x++) res[x] = v.look(lk.first + x);
+            }
+        };
+        auto batch_rows = [&](int64_t first, int64_t since) {
+            return std::min(std::min<int64_t>(rows - first, MAX_BATCH), std::max(FIRST_BATCH, since));
+        };
+        auto set_job = [&](Span st, Span lk) {
+            job_view = view();
+            job_store = st;
+            job_look = lk;
+            next_store.store(0, std::memory_order_relaxed);
+            next_look.store(0, std::memory_order_relaxed);
+        };
+        while (pool.size() > 1 && j < rows && group_size != max_rows) {
+            if (since_change < SERIAL_ROWS || rows - j < FIRST_BATCH) {
+                // right behind a merge the next one is often near: row by row (rows >= j are in no buffer)
+                const int64_t stop = std::min(rows, j + std::max<int64_t>(SERIAL_ROWS - since_change, rows - j < FIRST_BATCH ? rows - j : 0));
+                for (; j < stop && group_size != max_rows; j++) since_change = scan_row(j) ? 0 : since_change + 1;
                 continue;
             }
-            if (grouping[j] != -1) continue;
-            comparisons++;
-
-            const int64_t nb = pat.ptr[j + 1] - pat.ptr[j];
-            const bool b_empty = row_ptr[j + 1] == row_ptr[j];
-            float dist;
-            if (pattern_empty && b_empty) dist = 0.0f;
-            else if (pattern_empty || b_empty) dist = 1.0f;
-            else {
-                int64_t common = 0;
-                for (int64_t k = pat.ptr[j]; k < pat.ptr[j + 1]; k++) common += stamp[pat.blk[k]] == i;
-                const int64_t na = (int64_t)pattern.size();
-                // count_zeros weighting: blocks only in the group count once, blocks
-                // only in the row count group_size times (blocking.cpp:912-917)
-                const int64_t count = (na - common) + (nb - common) * group_size;
-                dist = (float)((2.0 * (double)count) / (double)(na * group_size + nb + count));
+            if (!looked.count) { // nothing looked at yet from j on: everybody looks
+                looked = Span{free_buffer(), j, batch_rows(j, since_change)};
+                set_job(stored, looked);
+                pool.run(job);
+                stored.count = 0;
             }
-            dist_cache[j] = dist;
-
-            if (dist <= tau) {
-                merges++;
-                grouping[j] = group_number;
-                merged_rows.push_back(j);
-                // merge_rows(pattern, row j): row j's columns, plus the pattern's
-                // columns below the largest column of row j that is <= max(pattern).
-                // An empty row j therefore empties the pattern.
-                int64_t cut = -1; // pattern blocks with id < cut survive
-                if (!b_empty && !pattern_empty) {
-                    const int64_t *bb = col_idx + row_ptr[j], *be = col_idx + row_ptr[j + 1];
-                    const int64_t *ub = std::upper_bound(bb, be, pattern_max);
-                    if (ub != bb) cut = *(ub - 1) / col_block;
+            // the helpers look at the rows behind this batch while its results are applied here
+            const int64_t behind = looked.first + looked.count;
+            ahead = Span{0, behind, behind < rows ? batch_rows(behind, since_change + looked.count) : 0};
+            {
+                Span keep = looked; // free_buffer() must not hand out the buffer being applied
+                ahead.buf = free_buffer();
+                looked = keep;
+            }
+            set_job(stored, ahead);
+            pool.start(job);
+            const float *res = results[looked.buf].data();
+            int64_t x = 0;
+            bool merged = false;
+            for (; x < looked.count; x++) {
+                const float r = res[x];
+                if (r < 0) continue;
+                comparisons++;
+                if (r > tau) {
+                    keep_candidate(looked.first + x, r);
+                    continue;
                 }
-                scratch.clear();
-                for (int32_t b : pattern) {
-                    if (b < cut) scratch.push_back(b);
-                    else stamp[b] = -1;
-                }
-                pattern.clear();
-                size_t a = 0;
-                int64_t k = pat.ptr[j];
-                while (a < scratch.size() || k < pat.ptr[j + 1]) {
-                    if (k >= pat.ptr[j + 1] || (a < scratch.size() && scratch[a] < pat.blk[k])) {
-                        pattern.push_back(scratch[a++]);
-                    } else {
-                        if (a < scratch.size() && scratch[a] == pat.blk[k]) a++;
-                        pattern.push_back(pat.blk[k++]);
-                    }
-                }
-                for (int32_t b : pattern) stamp[b] = i;
-                pattern_empty = b_empty;
-                pattern_max = b_empty ? -1 : col_idx[row_ptr[j + 1] - 1];
-                group_size++;
+                merged = true; // applied below, when the helpers no longer read the pattern
+                x++;
+                break;
+            }
+            pool.wait();
+            stored = Span{looked.buf, looked.first, x};
+            j = looked.first + x;
+            if (merged) {
+                merge(j - 1);
+                since_change = 0;
+                looked.count = 0; // what was looked at behind the merge saw the old pattern
             } else {
-                candidates.insert(dist, j);
-                const size_t room = (size_t)(max_rows - (int64_t)merged_rows.size());
-                if (candidates.size() > room) candidates.trim_from_end(room);
+                since_change += x;
+                looked = ahead;
             }
+        }
+        if (stored.count) { // distances of the last rows applied
+            const float *res = results[stored.buf].data();
+            for (int64_t x = 0; x < stored.count; x++)
+                if (res[x] != TAKEN) dist_cache[stored.first + x] = res[x];
         }
 
         if (group_size < max_rows) {

@@ -27,8 +27,7 @@ def test_fixtures_exist():
     assert len(FIXTURES) >= 10
 
 
-@pytest.mark.parametrize("path", FIXTURES, ids=[os.path.basename(p)[:-4] for p in FIXTURES])
-def test_grouping_permutation_and_counters_match_reference(smat, path):
+def check_fixture(smat, path):
     d = np.load(path)
     rows, cols = int(d["rows"]), int(d["cols"])
     for k, (cb, rb, tau) in enumerate(d["params"]):
@@ -39,6 +38,28 @@ def test_grouping_permutation_and_counters_match_reference(smat, path):
         nr, nc = reordered_edges(rows, d["row_ptr"], d["col_idx"], perm)
         assert np.array_equal(nr, d[f"reordered_rows_{k}"]) and np.array_equal(nc, d[f"reordered_cols_{k}"])
         assert np.array_equal(np.sort(perm), np.arange(rows))
+
+
+@pytest.mark.parametrize("path", FIXTURES, ids=[os.path.basename(p)[:-4] for p in FIXTURES])
+def test_grouping_permutation_and_counters_match_reference(smat, path):
+    check_fixture(smat, path)
+
+
+# The scan over the later rows runs in batches on several threads for large matrices (rows looked at in
+# parallel against the current pattern, results applied in row order up to the first merge).  These settings
+# send the small recorded matrices through that path: a few rows one by one behind every merge, then batches
+# of a handful of rows, so that merges fall into batches at every position.
+BATCHED = [dict(SMAT_REORDER_THREADS="4", SMAT_REORDER_SERIAL_ROWS="4", SMAT_REORDER_FIRST_BATCH="16"),
+           dict(SMAT_REORDER_THREADS="3", SMAT_REORDER_SERIAL_ROWS="1", SMAT_REORDER_FIRST_BATCH="8"),
+           dict(SMAT_REORDER_THREADS="2", SMAT_REORDER_SERIAL_ROWS="1", SMAT_REORDER_FIRST_BATCH="1")]
+
+
+@pytest.mark.parametrize("env", BATCHED, ids=["4x16", "3x8", "2x1"])
+@pytest.mark.parametrize("path", FIXTURES, ids=[os.path.basename(p)[:-4] for p in FIXTURES])
+def test_fixtures_through_the_batched_scan(smat, monkeypatch, path, env):
+    for k, v in env.items():
+        monkeypatch.setenv(k, v)
+    check_fixture(smat, path)
 
 
 def run_reference(tmp_path, r, c, cb, rb, tau):
@@ -90,6 +111,27 @@ def test_live_against_reference_program_stencil_32k_rows(smat, tmp_path):
     c = d["col_idx"].astype(np.int64)
     want = run_reference(tmp_path, r, c, 16, 16, 0.5)
     g, perm, _ = smat.reorder_rows(rows, int(d["K"]), d["row_ptr"].astype(np.int64), c, 16, 16, 0.5)
+    assert np.array_equal(g, want)
+
+
+@pytest.mark.skipif(ref_binary("Matrix_Blocking") is None, reason="oracle/_ref/Matrix_Blocking not built")
+@pytest.mark.parametrize("threads", ["1", "default", "4x64"])
+def test_live_against_reference_program_power_law_16k_rows(smat, tmp_path, monkeypatch, threads):
+    """R-MAT rows: the set of candidate rows of a group grows to thousands of entries (the reference trims it
+    only in some shapes of its tree), most rows are farther away than all of them, and distances repeat.  That
+    is where the shortcuts of the candidate set act (no-op insertions, the place of a key found from the last
+    key with the same distance), and 16,384 rows are enough for the threaded scan to switch itself on."""
+    if threads == "1":
+        monkeypatch.setenv("SMAT_REORDER_THREADS", "1")
+    elif threads == "4x64":
+        for k, v in dict(SMAT_REORDER_THREADS="4", SMAT_REORDER_SERIAL_ROWS="8", SMAT_REORDER_FIRST_BATCH="64").items():
+            monkeypatch.setenv(k, v)
+    d = gen.rmat(14, 16)
+    r = np.repeat(np.arange(int(d["M"])), np.diff(d["row_ptr"]))
+    c = d["col_idx"].astype(np.int64)
+    rows = int(r.max()) + 1  # rows behind the last nonempty one do not exist in an edge list
+    want = run_reference(tmp_path, r, c, 16, 16, 0.5)
+    g, perm, _ = smat.reorder_rows(rows, int(d["K"]), d["row_ptr"].astype(np.int64)[:rows + 1], c, 16, 16, 0.5)
     assert np.array_equal(g, want)
 
 
