@@ -237,6 +237,8 @@ def main():
     ap.add_argument("--no-verify", action="store_true", help="skip the check of sampled block rows against the CPU oracle")
     ap.add_argument("--no-attach-values", action="store_true",
                     help="do not let the plan look at the block values (the compact kernel, id 5, needs them)")
+    ap.add_argument("--b-row-major", action="store_true",
+                    help="hand B over row-major (B[k*N + n], the SMAT_B_ROW_MAJOR option) instead of the reference's column-major layout")
     ap.add_argument("--perm-file", default=None, help="npz with perm_rows / perm_cols / reorder_s (reordered R-MAT workload)")
     ap.add_argument("--calibration-copy-mib", type=int, default=0,
                     help="also run one plain device copy of this many MiB (a kernel of known HBM traffic, "
@@ -260,6 +262,8 @@ def main():
         return torch.from_numpy(np.ascontiguousarray(a).view(np.int16)).to(dev)
 
     vals, Bd = dev_i16(A["b_val"]), dev_i16(B)
+    if args.b_row_major:
+        Bd = Bd.view(N, K).t().contiguous()  # generators hand out the reference layout: N columns of K values
     rp = torch.from_numpy(A["b_row_ptr"].astype(np.int32)).to(dev)
     ci = torch.from_numpy(A["b_col_idx"].astype(np.int32)).to(dev)
     Cd = torch.zeros((M, N), dtype=torch.int16, device=dev)
@@ -271,7 +275,7 @@ def main():
         plan.attach_values(vals, rp, ci)  # one-off look at the zero pattern of the blocks (not timed, like the plan)
 
     def step():
-        smat_amd.spmm(vals, rp, ci, Bd, Cd, M, N, K, nnzb, plan=plan, kernel=args.kernel)
+        smat_amd.spmm(vals, rp, ci, Bd, Cd, M, N, K, nnzb, plan=plan, kernel=args.kernel, b_row_major=args.b_row_major)
 
     if args.calibration_copy_mib:
         src = torch.ones(args.calibration_copy_mib << 19, dtype=torch.int16, device=dev)
@@ -376,7 +380,7 @@ def main():
         "dtype": "f16",
         "data": "synthetic",
         "config": {"workload": args.workload, "M": M, "K": K, "N": N, "nnzb": nnzb, "block": 16,
-                   "c_dtype": "f16", "plan": None if plan is None else plan.info(),
+                   "c_dtype": "f16", "b_layout": "row-major" if args.b_row_major else "column-major (reference)", "plan": None if plan is None else plan.info(),
                    "pattern_sha256": sha256_of(A["b_row_ptr"].astype(np.int32), A["b_col_idx"].astype(np.int32)), **INFO},
         "roofline": roof,
         "verified": check_result,

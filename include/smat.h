@@ -249,6 +249,10 @@ int smat_csr_to_bcsr_device(size_t M, size_t K, const int32_t *row_ptr, const in
  *   stats     out, int64[4]: comparison_counter, merge_counter,
  *             VBR_nzblocks_count, VBR_longest_row (utilities.cpp:217-224,
  *             blocking.cpp:562-614); may be NULL
+ *
+ * Matrices of 16,384 rows and more are scanned on several threads (the hardware's
+ * count, at most 16; SMAT_REORDER_THREADS in the environment sets it, 1 = none):
+ * the output does not depend on the number of threads.
  */
 int smat_reorder_rows(int64_t rows, int64_t cols, const int64_t *row_ptr, const int64_t *col_idx,
                       int64_t col_block, int64_t row_block, float tau, int64_t *grouping,

@@ -135,6 +135,16 @@ def test_live_against_reference_program_power_law_16k_rows(smat, tmp_path, monke
     assert np.array_equal(g, want)
 
 
+def test_threaded_scan_gives_the_single_thread_result_at_32k_rows(smat, monkeypatch):
+    """Both passes of 32,768 R-MAT rows with the default thread count against one thread."""
+    d = gen.rmat(15, 16)
+    got = smat.reorder_csr(d["M"], d["K"], d["row_ptr"], d["col_idx"], 16, 16, 0.5, True)
+    monkeypatch.setenv("SMAT_REORDER_THREADS", "1")
+    want = smat.reorder_csr(d["M"], d["K"], d["row_ptr"], d["col_idx"], 16, 16, 0.5, True)
+    for a, b in zip(got, want):
+        assert np.array_equal(a, b)
+
+
 TWO_PASS = sorted(glob.glob(os.path.join(HERE, "golden", "reorder_two_pass", "*.npz")))
 
 
