@@ -32,6 +32,7 @@ struct smat_plan {
     int chunk = 0;
     int panel_tiles = 0;
     int n_items = 0, n_split_rows = 0, n_slots = 0;
+    int max_item_blocks = 0; // blocks of the longest row-wise work item
     WorkItem *d_items = nullptr;
     SplitRow *d_split = nullptr;
     float *d_workspace = nullptr;
@@ -157,6 +158,7 @@ extern "C" int smat_spmm_bcsr_f16_ex(const uint16_t *vals, const int32_t *row_pt
         a.split_rows = plan->d_split; a.n_split_rows = plan->n_split_rows;
         a.workspace = plan->d_workspace;
         a.panel_tiles = plan->panel_tiles;
+        a.max_item_blocks = plan->max_item_blocks;
         if (plan->d_bpack && N <= plan->n_cap && o.kernel != SMAT_KERNEL_ROWWISE_DIRECT) a.b_packed = plan->d_bpack;
     }
     int kernel = o.kernel;
@@ -203,6 +205,7 @@ extern "C" int smat_spmm_bcsr_f16_ex(const uint16_t *vals, const int32_t *row_pt
             d.items = plan->d_items_dense; d.n_items = plan->n_items_dense;
             d.split_rows = plan->d_split_dense; d.n_split_rows = plan->n_split_dense;
             d.workspace = plan->d_workspace_dense;
+            d.max_item_blocks = 0; // describes the whole matrix's list, not this one
             e = d.n_items ? launch_rowwise(d, static_cast<hipStream_t>(o.stream)) : hipSuccess;
         }
         if (e == hipSuccess) {
@@ -388,6 +391,7 @@ static int smat_plan_create_impl(smat_plan **out, const int32_t *row_ptr_host,
     std::vector<SplitRow> split;
     const int slot = rowwise_work_list(row_ptr_host, mb, chunk, nullptr, items, split);
     p->n_items = (int)items.size();
+    for (const WorkItem &wi : items) p->max_item_blocks = std::max(p->max_item_blocks, wi.end - wi.begin);
     p->panel_tiles = rowwise_panel_tiles(n_hint, 0, items.size());
     p->n_split_rows = (int)split.size();
     p->n_slots = slot;

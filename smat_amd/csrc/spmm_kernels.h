@@ -41,6 +41,7 @@ struct SpmmArgs {
     int n_split_rows;
     float *workspace; // device, n_slots * 16 * N floats
     uint16_t *b_packed; // device scratch of K * N halves, or nullptr: read the column-major B directly
+    int max_item_blocks; // blocks of the longest work item, 0 = not known (no plan): lets short rows take the short-row kernel
 };
 
 // Stream format and geometry of the sweep kernel: sweep_format.h (shared with the host-side plan builder).

@@ -214,6 +214,96 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 4))) voi
     }
 }
 
+// Small problems with short block rows (a band matrix: 9 blocks per row, 256 rows): the kernel above keeps the
+// operands of two block pairs in flight, so a row of five pairs costs four memory latencies one after the other
+// and the launch is over before the chip is busy.  Here a wavefront asks for the operands of all its pairs
+// (at most NP) at once: work item -> column indices -> operands, three latencies, then NP x TN MFMAs (pairs past
+// the end of the row multiply zeros).  Whole block rows only (dst < 0), B in place.
+template <int TN, bool C_F32, int NP>
+__global__ __launch_bounds__(256) void spmm_rowwise_short_kernel(
+    const uint16_t *__restrict__ vals, const int32_t *__restrict__ row_ptr, const int32_t *__restrict__ col_idx,
+    const uint16_t *__restrict__ B, void *__restrict__ Cout, const WorkItem *__restrict__ items, int n_items, int N,
+    long K, int n_panels)
+{
+    static_assert(TN == 2 || TN == 4, "panels of 32 or 64 columns");
+    constexpr int PANEL = 16 * TN;
+    const int lane = threadIdx.x & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+    const long w = (long)blockIdx.x * 4 + wave;
+    if (w >= (long)n_items * n_panels) return;
+    const int panel = (int)(w / n_items);
+    const int it = (int)(w - (long)panel * n_items);
+    int br, p0, p1;
+    if (items) {
+        const WorkItem wi = items[it];
+        br = wi.block_row; p0 = wi.begin; p1 = wi.end;
+    } else {
+        br = it; p0 = row_ptr[it]; p1 = row_ptr[it + 1];
+    }
+    br = __builtin_amdgcn_readfirstlane(br);
+    p0 = __builtin_amdgcn_readfirstlane(p0);
+    p1 = __builtin_amdgcn_readfirstlane(p1);
+    const int cnt = p1 - p0; // <= 2 * NP: the launcher has checked the work list
+    const int npair = (cnt + 1) >> 1;
+
+    const int i16 = lane & 15, g = lane >> 4, sel = g >> 1, kh = g & 1;
+    const int n0 = panel * PANEL;
+    f32x4 acc[TN];
+#pragma unroll
+    for (int t = 0; t < TN; t++) acc[t] = (f32x4){0.f, 0.f, 0.f, 0.f};
+    if (cnt > 0) { // uniform over the wavefront
+        long boff[TN];
+#pragma unroll
+        for (int t = 0; t < TN; t++) {
+            const int n = n0 + ncol_of<TN>(t, i16);
+            boff[t] = (long)(n < N ? n : 0) * K + kh * 8; // columns past N read column 0: never stored
+        }
+        const uint16_t *abase = vals + i16 * 16 + kh * 8;
+        const f16x8 zero8 = zero_f16x8();
+        const int myc = col_idx[p0 + (lane < cnt ? lane : cnt - 1)];
+        f16x8 a[NP], b[NP][TN];
+#pragma unroll
+        for (int j = 0; j < NP; j++) {
+            const int jj = j < npair ? j : npair - 1; // past the end: the last pair again, multiplied by zeros below
+            const int second = (2 * jj + 1 < cnt) ? 2 * jj + 1 : 2 * jj; // a single block pairs with itself
+            const int c0 = __builtin_amdgcn_readlane(myc, 2 * jj);
+            const int c1 = __builtin_amdgcn_readlane(myc, second);
+            const long pp = (long)p0 + (sel ? second : 2 * jj);
+            a[j] = load_f16x8(abase + pp * 256);
+            const long bc = sel ? c1 : c0;
+#pragma unroll
+            for (int t = 0; t < TN; t++) b[j][t] = load_f16x8(B + boff[t] + bc);
+        }
+        SMAT_ORDER_FENCE();
+#pragma unroll
+        for (int j = 0; j < NP; j++) {
+            f16x8 aj = a[j];
+            if (j >= npair) aj = zero8;
+            else if (2 * j + 1 >= cnt) aj = sel ? zero8 : aj; // single block: the upper K half contributes nothing
+#pragma unroll
+            for (int t = 0; t < TN; t++) acc[t] = __builtin_amdgcn_mfma_f32_16x16x32_f16(b[j][t], aj, acc[t], 0, 0, 0);
+        }
+    }
+    // acc[t][r] = C[br*16 + i16][n0 + ncol_of(t, 4*g + r)]: 4*TN consecutive columns per lane, as in the kernel above
+    const long m = (long)br * 16 + i16;
+    const int nbase = n0 + 4 * TN * g;
+    if (C_F32) {
+        float *crow = reinterpret_cast<float *>(Cout) + m * (long)N;
+#pragma unroll
+        for (int t = 0; t < TN; t++)
+            if (nbase + 4 * t < N) *reinterpret_cast<f32x4 *>(crow + nbase + 4 * t) = acc[t];
+    } else {
+        uint16_t *crow = reinterpret_cast<uint16_t *>(Cout) + m * (long)N;
+#pragma unroll
+        for (int t = 0; t < TN; t += 2) {
+            const f32x4 v0 = acc[t], v1 = acc[t + 1];
+            const f16x8 h = {(_Float16)v0[0], (_Float16)v0[1], (_Float16)v0[2], (_Float16)v0[3],
+                             (_Float16)v1[0], (_Float16)v1[1], (_Float16)v1[2], (_Float16)v1[3]};
+            if (nbase + 4 * t < N) *reinterpret_cast<f16x8 *>(crow + nbase + 4 * t) = h;
+        }
+    }
+}
+
 // Sums the fp32 partial tiles of every split block row in slot order and writes
 // the finished rows to C.  One thread per 4 consecutive columns of one row.
 template <bool C_F32>
@@ -311,9 +401,39 @@ int rowwise_panel_tiles(size_t N, int requested, size_t n_items)
     return 1;
 }
 
+// The short-row kernel: rows of at most 2 * SHORT_NP blocks, no split rows, B in place, few wavefronts.
+constexpr int SHORT_NP = 5;
+constexpr long SHORT_MAX_WAVES = 8192;
+
+template <int TN>
+static hipError_t launch_rowwise_short(const SpmmArgs &a, hipStream_t st)
+{
+    const int n_panels = (int)((a.N + 16 * TN - 1) / (16 * TN));
+    const long total = (long)a.n_items * n_panels;
+    if (total == 0) return hipSuccess;
+    dim3 grid((unsigned)((total + 3) / 4)), block(256);
+    if (a.c_f32)
+        hipLaunchKernelGGL((spmm_rowwise_short_kernel<TN, true, SHORT_NP>), grid, block, 0, st, a.vals, a.row_ptr, a.col_idx,
+                           a.B, a.C, a.items, a.n_items, (int)a.N, (long)a.K, n_panels);
+    else
+        hipLaunchKernelGGL((spmm_rowwise_short_kernel<TN, false, SHORT_NP>), grid, block, 0, st, a.vals, a.row_ptr, a.col_idx,
+                           a.B, a.C, a.items, a.n_items, (int)a.N, (long)a.K, n_panels);
+    return hipGetLastError();
+}
+
 hipError_t launch_rowwise(const SpmmArgs &a, hipStream_t st)
 {
     hipError_t e;
+    if (!a.b_packed && a.n_split_rows == 0 && a.max_item_blocks > 0 && a.max_item_blocks <= 2 * SHORT_NP && a.N >= 32 &&
+        (long)a.n_items * (long)((a.N + 31) / 32) <= SHORT_MAX_WAVES) {
+#ifndef SMAT_SHORT_TN
+        // 32-column panels while that still leaves the chip short of wavefronts, else 64
+        const bool narrow = (long)a.n_items * (long)((a.N + 63) / 64) < 2048;
+#else
+        const bool narrow = SMAT_SHORT_TN == 2;
+#endif
+        return narrow ? launch_rowwise_short<2>(a, st) : launch_rowwise_short<4>(a, st);
+    }
     if (a.b_packed) {
         dim3 grid((unsigned)((a.K + 63) / 64), (unsigned)((a.N + 63) / 64));
         hipLaunchKernelGGL(pack_b_kernel, grid, dim3(256), 0, st, a.B, a.b_packed, (int)a.N, (long)a.K);

@@ -175,6 +175,31 @@ def test_skewed_rows_with_and_without_plan(smat, cuda, oracle, lengths):
     assert rel_err_f32(c32, ref) <= TOL_F32
 
 
+@pytest.mark.parametrize("N", [32, 40, 64, 88, 128, 264])
+def test_short_rows_with_a_plan_match_the_oracle_and_the_general_kernel(smat, cuda, oracle, N):
+    """Rows of 0..10 blocks with a plan: the launcher takes the kernel that loads all operands of a row at once.
+    Odd and even lengths, single blocks, empty rows, partial last panel (N % 32 != 0 and N % 64 != 0); without
+    a plan the general row-wise kernel runs: same pairs, same order of the K = 32 steps, same bits."""
+    lengths = [0, 1, 2, 3, 4, 5, 6, 7, 8, 9, 10, 10, 1, 0, 9, 2, 10, 3, 0, 0, 7]
+    A = gen.random_bcsr(len(lengths), 12, 0.0, seed=77, row_lengths=lengths)
+    B = gen.dense_b(A["K"], N, seed=34)
+    ref = oracle_ref(oracle, A, B, N)
+    c_plan = gpu_spmm(smat, cuda, A, B, N, plan=True)
+    assert oracle.compare(c_plan, ref)[0] <= TOL_F16
+    assert np.array_equal(c_plan, gpu_spmm(smat, cuda, A, B, N, plan=False))
+    c32 = gpu_spmm(smat, cuda, A, B, N, plan=True, c_f32=True)
+    assert rel_err_f32(c32, ref) <= TOL_F32
+    assert np.array_equal(c32, gpu_spmm(smat, cuda, A, B, N, plan=False, c_f32=True))
+
+
+def test_rows_of_eleven_blocks_stay_with_the_general_kernel(smat, cuda, oracle):
+    lengths = [11, 3, 10, 0, 1]
+    A = gen.random_bcsr(len(lengths), 12, 0.0, seed=78, row_lengths=lengths)
+    N = 64
+    B = gen.dense_b(A["K"], N, seed=35)
+    assert oracle.compare(gpu_spmm(smat, cuda, A, B, N, plan=True), oracle_ref(oracle, A, B, N))[0] <= TOL_F16
+
+
 def test_plan_splits_long_rows(smat, cuda):
     lengths = [700] + [1] * 15
     A = gen.random_bcsr(16, 700, 0.0, seed=3, row_lengths=lengths)
