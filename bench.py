@@ -77,11 +77,31 @@ def verify_sample(A, B, N, C_bits, n_sample=24, tol=1e-3):
             "max_abs": float(f"{max_abs:.3e}"), "tolerance": tol, "ok": bool(rel <= tol and np.isfinite(rel))}
 
 
+GOLDEN_STRUCTURE = os.path.join(os.path.dirname(os.path.abspath(__file__)), "tests", "golden", "structure_hashes.json")
+
+
+def structure_against_golden(name, A):
+    """Compares the blocked structure (and the permutations of a reordered workload) with the hashes recorded
+    when the fixture file was made on another machine.  None if the workload has no entry."""
+    if not os.path.exists(GOLDEN_STRUCTURE):
+        return None
+    want = json.load(open(GOLDEN_STRUCTURE)).get(name)
+    if want is None:
+        return None
+    got = {"nnzb": int(A["nnzb"]),
+           "pattern_sha256": sha256_of(A["b_row_ptr"].astype(np.int32), A["b_col_idx"].astype(np.int32)),
+           "values_sha256": sha256_of(np.ascontiguousarray(A["b_val"]))}
+    if "perm_sha256" in want:
+        got["perm_sha256"] = INFO.get("perm_sha256")
+    return {"ok": all(got[k] == want[k] for k in got), "fixture": "tests/golden/structure_hashes.json",
+            "differs": [k for k in got if got[k] != want[k]]}
+
+
 INFO = {}  # facts about the generated workload that go into the config of the result line
 PERM_FILE = None
 
 
-def build_workload(name):
+def build_workload(name, want_b=True):
     from smat_amd import generators as gen
     import smat_amd
     if name == "block_pruned_8192_10pct_N4096":
@@ -142,7 +162,7 @@ def build_workload(name):
         N, bdist, bseed = 128, "uniform", 0xB0000003
     else:
         raise SystemExit(f"unknown workload {name}")
-    B = gen.dense_b(A["K"], N, seed=bseed, dist=bdist)
+    B = gen.dense_b(A["K"], N, seed=bseed, dist=bdist) if want_b else None
     return A, B, N
 
 
@@ -384,6 +404,7 @@ def main():
                    "pattern_sha256": sha256_of(A["b_row_ptr"].astype(np.int32), A["b_col_idx"].astype(np.int32)), **INFO},
         "roofline": roof,
         "verified": check_result,
+        "structure_vs_fixture": structure_against_golden(args.workload, A),
     }
     if not args.no_cpu_baseline:
         port = cpu_baseline(A, B, N)
@@ -392,6 +413,8 @@ def main():
         if ref is not None:
             out["cpu_baseline_all_cores"] = port
     print(json.dumps(out))
+    if out["structure_vs_fixture"] is not None and not out["structure_vs_fixture"]["ok"]:
+        raise SystemExit(f"bench.py: the blocked structure differs from the recorded one: {out['structure_vs_fixture']}")
     if check_result is not None and not check_result["ok"]:
         raise SystemExit(f"bench.py: the result of the last launch differs from the CPU oracle: {check_result}")
 
