@@ -12,22 +12,22 @@
 //  * Work.  A wavefront owns 8 of the 64 block rows (the plan picks which, so that the wavefronts have
 //    about the same work in every chunk) x 64 columns, 128 fp32 accumulator registers, and runs a
 //    host-built stream of ops.  One op = two blocks of one block row = one K = 32 step of
-//    v_mfma_f32_16x16x32_f16 per 16 columns (4 MFMAs).  The two blocks may sit in the same chunk or
-//    in two consecutive chunks (the ring keeps the previous stage), so few blocks stay unpaired.
+//    v_mfma_f32_16x16x32_f16 per 16 columns (4 MFMAs).  The two blocks may sit up to two
+//    listed chunks apart (three chunks are resident while the middle one is swept), so few blocks stay unpaired.
 //  * Interpreter.  The stream of a wavefront is threaded code (gen_sweep_loop.py, sweep_format.h): every 16-byte
 //    entry carries the offset of the code block that executes it, a block ends in a jump to the block of the
 //    next entry.  Blocks are specialised for the stream position modulo 8 (register sets), the block row
 //    (accumulators) and the s_waitcnt the op needs, so an op costs its 4 MFMAs, 4 LDS reads, one A load, the
 //    address arithmetic of the reads, two waits and the jump: 18 instructions.  Entries come in through scalar
-//    loads, two at a time, six positions ahead.
-//  * Pipeline.  The B operands of an op are read from LDS one position ahead (two register sets), its A
+//    loads, two at a time, five positions ahead.
+//  * Pipeline.  The B operands of an op are read from LDS two positions ahead (four register sets), its A
 //    operand (two neighbouring 512-byte blocks, one load straight into MFMA layout) comes from global memory
-//    five positions ahead (ring of eight).  Vector memory operations complete in order, so the number of
-//    younger ones at every wait is known when the plan is built: 5, or 9 when a marker issued its copies in
+//    three positions ahead (ring of four).  Vector memory operations complete in order, so the number of
+//    younger ones at every wait is known when the plan is built: 3, or 7 when a marker issued its copies in
 //    between.  A half of an MFMA that must not contribute (unpaired block) reads a 16 KiB region of zeros.
 //  * Accumulators live in a[0:127] and are touched by inline assembly only.
 //  * Synchronisation.  One barrier per chunk, in the marker entry that starts the chunk.  Marker of chunk c:
-//    the wavefront's own copies of chunk c (issued two markers earlier) have landed, barrier, then the copies
+//    the wavefront's own copies of chunk c+1 (issued one marker earlier) have landed, barrier, then the copies
 //    of chunk c+2 go into the stage that held chunk c-2.  The plan gives every wavefront at least four ops
 //    per chunk (filler ops that multiply zeros where it has fewer), so markers are at least five positions
 //    apart and every wavefront passes every barrier.
