@@ -16,21 +16,27 @@ Run after changing:
 
     python3 gen_sweep_loop.py > spmm_sweep_loop.inc
 
-Stream position i, J = i % 8.  Block of op i:
-    wait for the LDS reads of op i (set J % 4).  LDS reads return in order, so an even position waits until
-    four are left (those of op i + 1); an odd position waits for everything, which includes the descriptors
-    that the odd position before it asked for, and then loads the descriptors of ops i + 5 and i + 6
-    (scalar load of 32 bytes; scalar loads share the counter of the LDS reads but return in any order)
-    LDS reads of the B operands of op i + 2 (into set (J + 2) % 4)
-    load of the A operand of op i + AHEAD (into slot (J + AHEAD) % 4)
+Stream position i, J = i % 8.  Block of op i (default: --lds-ahead 1 --ahead 4):
+    even position: LDS reads of the B operands of op i + 1 (into set (J + 1) % 2), then a wait until only those
+    four are left: LDS reads return in order, so the reads of op i are in registers.  Scalar loads share the
+    counter and return in any order; with one of them under way the same wait holds for the reads of op i
+    (it then also waits for the first read of op i + 1 or for the scalar load, whichever comes first)
+    odd position: wait for everything (the reads of op i, and the descriptors that the odd position before it
+    asked for), scalar load of the descriptors of ops i + 7 and i + 8 (32 bytes), LDS reads of op i + 1
+    load of the A operand of op i + AHEAD (into slot (J + AHEAD) % 8)
     wait for the A operand of op i, 4 MFMAs, jump to op i + 1
+    The set that the reads of op i + 1 land in is the one the MFMAs of op i - 1 took their operands from a few
+    instructions earlier: an MFMA reads its A and B sources when it starts, LDS data arrives 64 clocks later
+    at the earliest.
+With --lds-ahead 2 every position issues the reads of op i + 2 (four sets), odd positions load the descriptors of
+ops i + 5 and i + 6, and the A ring has four slots (--ahead 2 or 3): the earlier pipeline, kept for comparison.
 Marker (first thing of every chunk but the first): own copies of the next chunk have landed, barrier,
 copies of the chunk after next, and the same read-ahead duties, no MFMAs.
 
-Registers (fixed, all listed as clobbers):
-    v40-v103   B operands, four sets of 4 tiles x 4 registers
-    v104-v119  A operands, ring of four
-    v120-v122  temporaries
+Registers (fixed, all listed as clobbers; --lds-ahead 1):
+    v40-v71    B operands, two sets of 4 tiles x 4 registers
+    v72-v103   A operands, ring of eight
+    v104-v106  temporaries
     s40-s71    descriptor ring, op i in slot i % 8: w0 w1 w2 w3
     s72-s85    state: descriptor pointer, code base, chunk counter, next chunk id, chunk list pointer,
                temporaries, jump target
@@ -40,12 +46,16 @@ Registers (fixed, all listed as clobbers):
 import argparse
 
 ap = argparse.ArgumentParser()
-ap.add_argument("--ahead", type=int, default=3, help="A operands are loaded this many ops ahead (2 or 3: ring of four, descriptors arrive two positions before their first use)")
+ap.add_argument("--ahead", type=int, default=4, help="A operands are loaded this many ops ahead (2..5 with --lds-ahead 1: ring of eight; 2..3 with --lds-ahead 2: ring of four)")
+ap.add_argument("--lds-ahead", type=int, default=1, help="B operands are read from LDS this many positions ahead: 2 (four register sets, A ring of four) or 1 (two sets, A ring of eight, --ahead up to 5)")
 ap.add_argument("--ablate", default="", help="timing experiments only, wrong results: any of a,copy,barrier,mfma,bread,vm")
 args = ap.parse_args()
 AHEAD = args.ahead
+LB = args.lds_ahead
 ABL = set(x for x in args.ablate.split(",") if x)
-assert 2 <= AHEAD <= 3
+assert LB in (1, 2)
+BSETS, ARING = (4, 4) if LB == 2 else (2, 8)
+assert 2 <= AHEAD <= (3 if LB == 2 else 5)
 
 RING = 8
 BLOCK_BYTES = 128                        # SWEEP_BLOCK_BYTES
@@ -57,9 +67,13 @@ MIN_OPS = max(AHEAD - 1, COPIES)
 VM_MARK = MIN_OPS + 1      # a marker's copies of one marker ago are older than the A loads of the MIN_OPS + 1 positions since
 
 S_RING0 = 40
+DESC_AHEAD = 5 if LB == 2 else 7   # an odd position loads the descriptors of ops i + DESC_AHEAD and the one after
 S_DP, S_BASE, S_CUR, S_NEXTK, S_CP, S_T0, S_T1, S_JMP = 72, 74, 76, 77, 78, 80, 81, 84
 S_LAST = 85
-V_B0, V_A0, V_T0, V_T1, V_COPY = 40, 104, 120, 121, 122
+V_B0 = 40
+V_A0 = V_B0 + 16 * BSETS
+V_T0 = V_A0 + 4 * ARING
+V_T1, V_COPY = V_T0 + 1, V_T0 + 2
 
 
 def ring(slot, word):
@@ -67,12 +81,12 @@ def ring(slot, word):
 
 
 def bset(s, t):
-    b = V_B0 + 16 * (s % 4) + 4 * t
+    b = V_B0 + 16 * (s % BSETS) + 4 * t
     return f"v[{b}:{b + 3}]"
 
 
 def aslot(d):
-    b = V_A0 + 4 * (d % 4)
+    b = V_A0 + 4 * (d % ARING)
     return f"v[{b}:{b + 3}]"
 
 
@@ -107,6 +121,21 @@ def a_load(slot):
 
 def top_wait(J):
     """B operands of op i are in registers.  Odd positions: everything asked for so far is, and the next two descriptors are asked for."""
+    if LB == 1:
+        # reads one position ahead: an even position asks for those of op i + 1 first and waits until only they are
+        # left; an odd position waits for everything (reads of op i, descriptors asked for two positions ago),
+        # asks for two descriptors and then for the reads of op i + 1
+        if J % 2 == 0:
+            b_reads(J + 1, J + 1)
+            emit("s_waitcnt lgkmcnt(4)")
+            return
+        emit("s_waitcnt lgkmcnt(0)")
+        s0 = S_RING0 + 4 * ((J + DESC_AHEAD) % RING)
+        emit(f"s_load_dwordx8 s[{s0}:{s0 + 7}], s[{S_DP}:{S_DP + 1}], 0x0")
+        emit(f"s_add_u32 s{S_DP}, s{S_DP}, 32")
+        emit(f"s_addc_u32 s{S_DP + 1}, s{S_DP + 1}, 0")
+        b_reads(J + 1, J + 1)
+        return
     if J % 2 == 0:
         emit("s_waitcnt lgkmcnt(4)")
         return
@@ -127,7 +156,8 @@ def op_block(J, r, v):
     k = (J * 8 + r) * 2 + v
     label(f"Lb{k}")
     top_wait(J)
-    b_reads(J + 2, J + 2)
+    if LB == 2:
+        b_reads(J + 2, J + 2)
     a_load(J + AHEAD)
     if "vm" not in ABL:
         emit(f"s_waitcnt vmcnt({AHEAD + COPIES * v})")
@@ -169,7 +199,8 @@ def marker_block(J):
     emit(f"s_load_dword s{S_NEXTK}, s[{S_CP}:{S_CP + 1}], 0x0")   # id of chunk cur + 3, for the next marker
     emit(f"s_add_u32 s{S_CP}, s{S_CP}, 4")
     emit(f"s_addc_u32 s{S_CP + 1}, s{S_CP + 1}, 0")
-    b_reads(J + 2, J + 2)
+    if LB == 2:
+        b_reads(J + 2, J + 2)
     a_load(J + AHEAD)
     jump(J + 1)
     emit(f".org Lb0_%= + {MARK_BASE + (J + 1) * MARK_BYTES}")
@@ -179,8 +210,11 @@ def marker_block(J):
 emit(f"s_mov_b32 s{S_DP}, %[op_lo]")
 emit(f"s_mov_b32 s{S_DP + 1}, %[op_hi]")
 emit(f"s_load_dwordx16 s[{S_RING0}:{S_RING0 + 15}], s[{S_DP}:{S_DP + 1}], 0x0")
-emit(f"s_load_dwordx8 s[{S_RING0 + 16}:{S_RING0 + 23}], s[{S_DP}:{S_DP + 1}], 0x40")
-emit(f"s_add_u32 s{S_DP}, s{S_DP}, 96")
+if LB == 2:
+    emit(f"s_load_dwordx8 s[{S_RING0 + 16}:{S_RING0 + 23}], s[{S_DP}:{S_DP + 1}], 0x40")
+else:
+    emit(f"s_load_dwordx16 s[{S_RING0 + 16}:{S_RING0 + 31}], s[{S_DP}:{S_DP + 1}], 0x40")
+emit(f"s_add_u32 s{S_DP}, s{S_DP}, {96 if LB == 2 else 128}")
 emit(f"s_addc_u32 s{S_DP + 1}, s{S_DP + 1}, 0")
 emit(f"s_mov_b32 s{S_CP}, %[chunk_lo]")
 emit(f"s_mov_b32 s{S_CP + 1}, %[chunk_hi]")
@@ -195,7 +229,8 @@ emit(f"s_waitcnt vmcnt({AHEAD})")                     # the copies of chunks 0, 
 if "barrier" not in ABL:
     emit("s_barrier")
 b_reads(0, 0)
-b_reads(1, 1)
+if LB == 2:
+    b_reads(1, 1)
 emit(f"s_getpc_b64 s[{S_BASE}:{S_BASE + 1}]")
 label("Lpc")
 emit(f"s_add_u32 s{S_BASE}, s{S_BASE}, Lb0_%=-Lpc_%=")
@@ -212,7 +247,8 @@ label("Lend")                                         # offset END_OFF: the desc
 emit("s_waitcnt vmcnt(0) lgkmcnt(0)")
 
 clob = [f'"v{i}"' for i in range(V_B0, V_COPY + 1)] + [f'"s{i}"' for i in range(S_RING0, S_LAST + 1)] + ['"vcc"', '"scc"', '"memory"']
-print(f"// generated by gen_sweep_loop.py --ahead {AHEAD}" + (f" --ablate {args.ablate}" if ABL else "") + "; do not edit")
+print(f"// generated by gen_sweep_loop.py --ahead {AHEAD} --lds-ahead {LB}" + (f" --ablate {args.ablate}" if ABL else "") + "; do not edit")
+print(f"static_assert(SWEEP_LDS_AHEAD == {LB}, \"regenerate spmm_sweep_loop.inc\");")
 print(f"static_assert(SWEEP_AHEAD == {AHEAD} && SWEEP_BLOCK_BYTES == {BLOCK_BYTES} && SWEEP_MARK_BASE == {MARK_BASE} && "
       f"SWEEP_MARK_BYTES == {MARK_BYTES} && SWEEP_END_OFF == {END_OFF}, \"regenerate spmm_sweep_loop.inc\");")
 print("asm volatile(")

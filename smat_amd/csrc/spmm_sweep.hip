@@ -19,11 +19,11 @@
 //    next entry.  Blocks are specialised for the stream position modulo 8 (register sets), the block row
 //    (accumulators) and the s_waitcnt the op needs, so an op costs its 4 MFMAs, 4 LDS reads, one A load, the
 //    address arithmetic of the reads, two waits and the jump: 18 instructions.  Entries come in through scalar
-//    loads, two at a time, five positions ahead.
-//  * Pipeline.  The B operands of an op are read from LDS two positions ahead (four register sets), its A
+//    loads, two at a time, seven positions ahead.
+//  * Pipeline.  The B operands of an op are read from LDS one position ahead (two register sets), its A
 //    operand (two neighbouring 512-byte blocks, one load straight into MFMA layout) comes from global memory
-//    three positions ahead (ring of four).  Vector memory operations complete in order, so the number of
-//    younger ones at every wait is known when the plan is built: 3, or 7 when a marker issued its copies in
+//    four positions ahead (ring of eight).  Vector memory operations complete in order, so the number of
+//    younger ones at every wait is known when the plan is built: 4, or 8 when a marker issued its copies in
 //    between.  A half of an MFMA that must not contribute (unpaired block) reads a 16 KiB region of zeros.
 //  * Accumulators live in a[0:127] and are touched by inline assembly only.
 //  * Synchronisation.  One barrier per chunk, in the marker entry that starts the chunk.  Marker of chunk c:

@@ -13,9 +13,13 @@ constexpr int SWEEP_G = SWEEP_RW * SWEEP_WAVES; // 64 block rows per workgroup
 constexpr int SWEEP_S = 16;      // block columns (slabs) per K chunk
 constexpr int SWEEP_STAGES = 4;  // chunks resident in LDS
 #ifndef SWEEP_AHEAD_VALUE
-#define SWEEP_AHEAD_VALUE 3
+#define SWEEP_AHEAD_VALUE 4
 #endif
 constexpr int SWEEP_AHEAD = SWEEP_AHEAD_VALUE; // an A operand is loaded this many stream positions before its op
+#ifndef SWEEP_LDS_AHEAD_VALUE
+#define SWEEP_LDS_AHEAD_VALUE 1
+#endif
+constexpr int SWEEP_LDS_AHEAD = SWEEP_LDS_AHEAD_VALUE; // the B operands of an op are read from LDS this many stream positions before it
 constexpr int SWEEP_COPIES = 4;  // copy instructions per wavefront and chunk
 constexpr int SWEEP_MIN_OPS = SWEEP_AHEAD - 1 > SWEEP_COPIES ? SWEEP_AHEAD - 1 : SWEEP_COPIES; // ops per wavefront and chunk: two markers are at least AHEAD positions apart, and a marker finds the copies of the marker before it older than the A loads of the MIN_OPS + 1 positions since
 constexpr int SWEEP_OP_PAD = 16;   // descriptors after the end of the last stream (loaded ahead, never executed)

@@ -323,6 +323,12 @@ static int smat_internal_sweep_plan_impl(const int32_t *row_ptr, const int32_t *
     return SMAT_OK;
 }
 
+// Test hook: the pipeline depths this build was compiled with {A read-ahead, LDS read-ahead, minimum ops per chunk, copies per marker}.
+extern "C" void smat_internal_sweep_params(int32_t *out)
+{
+    out[0] = smat::SWEEP_AHEAD; out[1] = smat::SWEEP_LDS_AHEAD; out[2] = smat::SWEEP_MIN_OPS; out[3] = smat::SWEEP_COPIES;
+}
+
 extern "C" int smat_internal_sweep_plan(const int32_t *row_ptr, const int32_t *col_idx, size_t M, size_t K,
                                          int32_t **rg_chunk_ptr, int32_t **chunk_ids, int32_t **op_ptr,
                                          uint32_t **ops, int32_t **row_map, int64_t *counts)

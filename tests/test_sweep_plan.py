@@ -14,8 +14,10 @@ from smat_amd import generators as gen
 from smat_amd._lib import lib
 
 G, RW, WAVES, S, STAGES = 64, 8, 8, 16, 4
-AHEAD, COPIES, MIN_OPS = 3, 4, 4
-PB = 2  # the LDS reads of an op are issued this many stream positions before it
+_params = (C.c_int32 * 4)()
+lib.smat_internal_sweep_params(_params)
+AHEAD, PB, MIN_OPS, COPIES = (int(x) for x in _params)  # A read-ahead, LDS read-ahead (positions), ops per chunk, copies per marker
+assert (AHEAD, PB) in ((3, 2), (4, 1), (5, 1)) and MIN_OPS == max(AHEAD - 1, COPIES)
 ZERO_OFF = 131072
 BLOCK_BYTES, MARK_BASE, MARK_BYTES = 128, 16384, 512
 END_OFF = MARK_BASE + 8 * MARK_BYTES
@@ -95,7 +97,9 @@ def replay(plan, A, Bd):
             period = []  # chunk period of every stream position (a marker belongs to the chunk it opens)
             for i, (w0, w1, w2, w3) in enumerate(tuple(int(x) for x in e) for e in ops):
                 assert not ended, "entries after the end of a stream"
-                period.append(cur + 1 if END_OFF > w3 >= MARK_BASE else cur)
+                # what the LDS reads issued at this position may see: a marker issues its reads behind its barrier when
+                # they are two positions ahead (it then belongs to the chunk it opens), before it when one ahead
+                period.append(cur + 1 if END_OFF > w3 >= MARK_BASE and PB == 2 else cur)
                 if w3 == END_OFF:
                     assert (w0, w1, w2) == (0, ZERO_OFF, 0)
                     ended = True
