@@ -48,6 +48,7 @@ import argparse
 ap = argparse.ArgumentParser()
 ap.add_argument("--ahead", type=int, default=4, help="A operands are loaded this many ops ahead (2..5 with --lds-ahead 1: ring of eight; 2..3 with --lds-ahead 2: ring of four)")
 ap.add_argument("--lds-ahead", type=int, default=1, help="B operands are read from LDS this many positions ahead: 2 (four register sets, A ring of four) or 1 (two sets, A ring of eight, --ahead up to 5)")
+ap.add_argument("--block-bytes", type=int, default=128, help="size of an op block's slot (SWEEP_BLOCK_BYTES)")
 ap.add_argument("--ablate", default="", help="timing experiments only, wrong results: any of a,copy,barrier,mfma,bread,vm")
 args = ap.parse_args()
 AHEAD = args.ahead
@@ -58,7 +59,7 @@ BSETS, ARING = (4, 4) if LB == 2 else (2, 8)
 assert 2 <= AHEAD <= (3 if LB == 2 else 5)
 
 RING = 8
-BLOCK_BYTES = 128                        # SWEEP_BLOCK_BYTES
+BLOCK_BYTES = args.block_bytes           # SWEEP_BLOCK_BYTES
 MARK_BASE = 8 * 8 * 2 * BLOCK_BYTES      # SWEEP_MARK_BASE: after the 128 op blocks
 MARK_BYTES = 512                         # SWEEP_MARK_BYTES
 END_OFF = MARK_BASE + 8 * MARK_BYTES     # SWEEP_END_OFF
@@ -159,6 +160,13 @@ def op_block(J, r, v):
     if LB == 2:
         b_reads(J + 2, J + 2)
     a_load(J + AHEAD)
+    for x in ABL:   # experiments on instruction fetch: padlit4 = 4 scalar moves with a literal (32 bytes), pad4 / pad8 = without (16 / 32 bytes)
+        if x.startswith("padlit"):
+            for _ in range(int(x[6:])):
+                emit("s_mov_b32 s86, 0x12345678")
+        elif x.startswith("pad"):
+            for _ in range(int(x[3:])):
+                emit("s_mov_b32 s86, 1")
     if "vm" not in ABL:
         emit(f"s_waitcnt vmcnt({AHEAD + COPIES * v})")
     for t in range(4):
@@ -246,7 +254,7 @@ for J in range(8):
 label("Lend")                                         # offset END_OFF: the descriptor after the last op jumps here
 emit("s_waitcnt vmcnt(0) lgkmcnt(0)")
 
-clob = [f'"v{i}"' for i in range(V_B0, V_COPY + 1)] + [f'"s{i}"' for i in range(S_RING0, S_LAST + 1)] + ['"vcc"', '"scc"', '"memory"']
+clob = [f'"v{i}"' for i in range(V_B0, V_COPY + 1)] + [f'"s{i}"' for i in range(S_RING0, S_LAST + 2)] + ['"vcc"', '"scc"', '"memory"']
 print(f"// generated by gen_sweep_loop.py --ahead {AHEAD} --lds-ahead {LB}" + (f" --ablate {args.ablate}" if ABL else "") + "; do not edit")
 print(f"static_assert(SWEEP_LDS_AHEAD == {LB}, \"regenerate spmm_sweep_loop.inc\");")
 print(f"static_assert(SWEEP_AHEAD == {AHEAD} && SWEEP_BLOCK_BYTES == {BLOCK_BYTES} && SWEEP_MARK_BASE == {MARK_BASE} && "

@@ -45,7 +45,10 @@ struct SweepOp {
 };
 constexpr uint32_t SWEEP_STAGE_BYTES = 32768;
 constexpr uint32_t SWEEP_ZERO_OFF = SWEEP_STAGES * SWEEP_STAGE_BYTES; // 131072
-constexpr uint32_t SWEEP_BLOCK_BYTES = 128;
+#ifndef SWEEP_BLOCK_BYTES_VALUE
+#define SWEEP_BLOCK_BYTES_VALUE 128
+#endif
+constexpr uint32_t SWEEP_BLOCK_BYTES = SWEEP_BLOCK_BYTES_VALUE;
 constexpr uint32_t SWEEP_MARK_BASE = 8 * 8 * 2 * SWEEP_BLOCK_BYTES;   // 16384
 constexpr uint32_t SWEEP_MARK_BYTES = 512;
 constexpr uint32_t SWEEP_END_OFF = SWEEP_MARK_BASE + 8 * SWEEP_MARK_BYTES;
