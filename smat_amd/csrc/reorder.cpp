@@ -694,18 +694,27 @@ std::vector<int64_t> keeper_grouping(int64_t rows, const int64_t *row_ptr, const
             const float *res = results[looked.buf].data();
             int64_t x = 0;
             bool merged = false;
+            // no merge inside the loop: the room for candidates stays what it is
+            const size_t room = (size_t)(max_rows - (int64_t)merged_rows.size());
+            const bool odd_room = room & 1;
+            int64_t compared = 0;
             for (; x < looked.count; x++) {
                 const float r = res[x];
                 if (r < 0) continue;
-                comparisons++;
+                compared++;
                 if (r > tau) {
-                    keep_candidate(looked.first + x, r);
+                    const int64_t row = looked.first + x;
+                    // most rows are farther than every candidate kept so far: see insert_then_trim_is_noop
+                    if (odd_room && candidates.size() >= room && candidates.insert_then_trim_is_noop(r, row)) continue;
+                    candidates.insert(r, row);
+                    if (candidates.size() > room) candidates.trim_from_end(room);
                     continue;
                 }
                 merged = true; // applied below, when the helpers no longer read the pattern
                 x++;
                 break;
             }
+            comparisons += compared;
             pool.wait();
             stored = Span{looked.buf, looked.first, x};
             j = looked.first + x;
