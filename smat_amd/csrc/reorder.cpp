@@ -683,12 +683,7 @@ std::vector<int64_t> keeper_grouping(int64_t rows, const int64_t *row_ptr, const
             }
             // the helpers look at the rows behind this batch while its results are applied here
             const int64_t behind = looked.first + looked.count;
-            ahead = Span{0, behind, behind < rows ? batch_rows(behind, since_change + looked.count) : 0};
-            {
-                Span keep = looked; // free_buffer() must not hand out the buffer being applied
-                ahead.buf = free_buffer();
-                looked = keep;
-            }
+            ahead = Span{free_buffer(), behind, behind < rows ? batch_rows(behind, since_change + looked.count) : 0};
             set_job(stored, ahead);
             pool.start(job);
             const float *res = results[looked.buf].data();
