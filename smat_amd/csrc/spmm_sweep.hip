@@ -102,7 +102,7 @@ __global__ __launch_bounds__(THREADS) void spmm_sweep_kernel(
     const uint16_t *__restrict__ vals, const uint16_t *__restrict__ B, void *__restrict__ Cout,
     const int32_t *__restrict__ rg_chunk_ptr, const int32_t *__restrict__ chunk_ids,
     const int32_t *__restrict__ op_ptr, const SweepOp *__restrict__ ops, const int32_t *__restrict__ row_map, int N, long K, int n_rg, int n_panels,
-    uint32_t vals_bytes)
+    uint32_t vals_bytes, int n_vb)
 {
     extern __shared__ __align__(16) unsigned char lds[];
 
@@ -113,15 +113,18 @@ __global__ __launch_bounds__(THREADS) void spmm_sweep_kernel(
     // Tile order: blocks of 4 row groups; inside a block panel-major, row group fastest.  Each XCD
     // (workgroup id modulo 8) takes a contiguous eighth, so the 32 workgroups it runs at a time are
     // 4 row groups x 8 panels: every A block is wanted by 8 of them, every B chunk by 4.
+    // A workgroup takes the tiles vb = blockIdx.x, blockIdx.x + gridDim.x, ... of the virtual grid n_vb.
     const int total = n_rg * n_panels;
-    const int per_xcd = gridDim.x >> 3;
-    const int tile = (blockIdx.x & 7) * per_xcd + (blockIdx.x >> 3);
-    if (tile >= total) return;
+    const int per_xcd = n_vb >> 3;
 #ifndef SWEEP_RGB
 #define SWEEP_RGB 4
 #endif
     constexpr int RGB = SWEEP_RGB;
     const int n_blk = (n_rg + RGB - 1) / RGB;
+    bool zeros_written = false;
+  for (int vb = blockIdx.x; vb < n_vb; vb += gridDim.x) {
+    const int tile = (vb & 7) * per_xcd + (vb >> 3);
+    if (tile >= total) continue;
     int gb = tile / (RGB * n_panels);
     gb = gb < n_blk - 1 ? gb : n_blk - 1;
     const int rem = tile - gb * RGB * n_panels;
@@ -186,14 +189,16 @@ __global__ __launch_bounds__(THREADS) void spmm_sweep_kernel(
             lds_copy(voff, sb3, dst0 + 3072u);
         };
         // ---- entry: chunks 0, 1, 2 on their way, the region of zeros written ----
+        if (zeros_written) __syncthreads(); // a later tile of this workgroup: everybody has left the stages of the tile before
         issue_copies(0);
         if (n_chunks > 1) issue_copies(1);
         if (n_chunks > 2) issue_copies(2);
-        {
+        if (!zeros_written) {
             i32x4 *zero = reinterpret_cast<i32x4 *>(lds + NS * STAGE_BYTES);
             zero[tid] = i32x4{0, 0, 0, 0};
             zero[tid + THREADS] = i32x4{0, 0, 0, 0};
             static_assert(ZERO_BYTES == 2 * THREADS * 16, "two 16-byte stores per lane fill the region of zeros");
+            zeros_written = true;
         }
         asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
 
@@ -240,6 +245,7 @@ __global__ __launch_bounds__(THREADS) void spmm_sweep_kernel(
     store_row(std::integral_constant<int, 2>{}); store_row(std::integral_constant<int, 3>{});
     store_row(std::integral_constant<int, 4>{}); store_row(std::integral_constant<int, 5>{});
     store_row(std::integral_constant<int, 6>{}); store_row(std::integral_constant<int, 7>{});
+  }
 }
 
 hipError_t launch_sweep(const SweepArgs &a, hipStream_t st)
@@ -258,15 +264,31 @@ hipError_t launch_sweep(const SweepArgs &a, hipStream_t st)
     wgs = (wgs + 7) / 8 * 8;
     if (wgs == 0) return hipSuccess;
     if (wgs > 0x7fffffffL) return hipErrorInvalidValue;
-    dim3 grid((unsigned)wgs), block(THREADS);
+    // One workgroup per CU at a time (144 KiB of LDS, 512 threads x 256 registers): with more tiles than CUs a
+    // workgroup keeps its CU and takes its tiles one after the other, which saves the dispatch of the later
+    // ones and lets the stores of a tile drain while the next one fetches its first chunks.
+    long launched = wgs;
+#ifdef SWEEP_PERSISTENT_GRID
+    if (SWEEP_PERSISTENT_GRID > 0 && launched > SWEEP_PERSISTENT_GRID) launched = SWEEP_PERSISTENT_GRID;
+#else
+    {
+        int dev = 0, cus = 0;
+        if (hipGetDevice(&dev) == hipSuccess &&
+            hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev) == hipSuccess && cus >= 8) {
+            const long resident = cus / 8 * 8; // workgroup ids are dealt round-robin to the 8 XCDs: keep a multiple of 8
+            if (launched > resident) launched = resident;
+        }
+    }
+#endif
+    dim3 grid((unsigned)launched), block(THREADS);
     if (a.c_f32)
         hipLaunchKernelGGL((spmm_sweep_kernel<true>), grid, block, lds_bytes, st, a.vals, a.B, a.C,
                            a.rg_chunk_ptr, a.chunk_ids, a.op_ptr, a.ops, a.row_map, (int)a.N, (long)a.K,
-                           a.n_rg, n_panels, (uint32_t)(a.nnzb * 512));
+                           a.n_rg, n_panels, (uint32_t)(a.nnzb * 512), (int)wgs);
     else
         hipLaunchKernelGGL((spmm_sweep_kernel<false>), grid, block, lds_bytes, st, a.vals, a.B, a.C,
                            a.rg_chunk_ptr, a.chunk_ids, a.op_ptr, a.ops, a.row_map, (int)a.N, (long)a.K,
-                           a.n_rg, n_panels, (uint32_t)(a.nnzb * 512));
+                           a.n_rg, n_panels, (uint32_t)(a.nnzb * 512), (int)wgs);
     return hipGetLastError();
 }
 
