@@ -222,6 +222,8 @@ SWEEP = 2
     (70, 20, 0.30, 72),     # N just above one panel
     (130, 160, 1.00, 64),   # dense, ten chunks: 64 ops per wavefront and chunk, several descriptor windows
     (200, 300, 0.12, 192),  # four row groups, 19 chunks: the ring of stages wraps several times
+    (64, 16, 0.50, 38408),  # 601 tiles on 256 CUs: a workgroup takes two or three tiles one after the other, last panel partial
+    (140, 20, 0.30, 12808), # three row groups x 201 panels = 603 tiles, rounded up to 608 workgroup ids: ids without a tile
 ])
 def test_sweep_kernel_matches_oracle(smat, cuda, oracle, mb, kb, density, N):
     A = gen.random_bcsr(mb, kb, density, seed=1000 + mb + kb)
