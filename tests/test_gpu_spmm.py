@@ -376,6 +376,31 @@ def test_config4_block_pruned_full_size_sampled_rows(smat, cuda, oracle):
     assert d <= 2e-3 * np.abs(C.view(np.float16).astype(np.float32)).max()
 
 
+def test_sweep_kernel_gives_the_same_bits_on_every_launch(smat, cuda):
+    """The sweep kernel reuses an operand register set for the next op's LDS reads a few instructions after the
+    MFMAs that read it were issued, and a workgroup reuses its LDS stages for its next tile: a late read or an
+    early overwrite would show as launches of the same product that differ.  Headline size, 24 launches with one
+    plan into fresh outputs, all compared bit for bit with the first."""
+    import torch
+    A = gen.block_pruned(8192, 0.10, 0.02)
+    N = 4096
+    B = gen.dense_b(8192, N, seed=0xB0000004, dist="normal")
+    M, K, nnzb = A["M"], A["K"], A["nnzb"]
+    vals, Bd = to_dev(torch, A["b_val"], cuda), to_dev(torch, B, cuda)
+    rp, ci = to_dev(torch, A["b_row_ptr"].astype(np.int32), cuda), to_dev(torch, A["b_col_idx"].astype(np.int32), cuda)
+    p = smat.Plan(A["b_row_ptr"], M, K, nnzb, N, col_idx_host=A["b_col_idx"], kernel=SWEEP)
+    first = None
+    for launch in range(24):
+        C = torch.full((M, N), 0x7E00, dtype=torch.int16, device=cuda)
+        smat.spmm(vals, rp, ci, Bd, C, M, N, K, nnzb, plan=p, kernel=SWEEP)
+        torch.cuda.synchronize()
+        if first is None:
+            first = C
+        else:
+            assert torch.equal(C, first), f"launch {launch} differs from the first"
+    p.close()
+
+
 COMPACT = 5
 
 
