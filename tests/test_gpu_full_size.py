@@ -134,3 +134,30 @@ def test_mixed_dispatch_full_size(smat, cuda, oracle):
     assert info["sweep_ops"] > 0 and info["mixed_dense_items"] == 0  # sweep, not row-wise, for the dense rows
     mb = A["M"] // 16
     check_sampled(oracle, A, B, N, C, sample_rows(mb, 16, extra=(mb // 2 - 1, mb // 2, mb // 2 + 1)))
+
+
+def test_config4_sweep_kernel_full_size_linearity_and_more_rows(smat, cuda, oracle):
+    """Headline config through the plan's choice (the sweep kernel): 40 sampled block rows against the oracle
+    (first and last of every row group among them), and A (2 B) = 2 (A B) bit for bit over the whole result."""
+    import torch
+    A = gen.block_pruned(8192, 0.10, 0.02)
+    N = 4096
+    M, K, nnzb = A["M"], A["K"], A["nnzb"]
+    B = gen.dense_b(K, N, seed=0xB0000004, dist="normal")
+    B2 = (B.view(np.float16) * np.float16(2)).view(np.uint16)
+    vals, Bd, B2d = to_dev(torch, A["b_val"], cuda), to_dev(torch, B, cuda), to_dev(torch, B2, cuda)
+    rp, ci = to_dev(torch, A["b_row_ptr"].astype(np.int32), cuda), to_dev(torch, A["b_col_idx"].astype(np.int32), cuda)
+    plan = smat.Plan(A["b_row_ptr"], M, K, nnzb, N, col_idx_host=A["b_col_idx"])
+    assert plan.info()["kernel"] == 2
+    C = torch.full((M, N), 0x7E00, dtype=torch.int16, device=cuda)
+    smat.spmm(vals, rp, ci, Bd, C, M, N, K, nnzb, plan=plan)
+    C2 = torch.full((M, N), 0x7E00, dtype=torch.int16, device=cuda)
+    smat.spmm(vals, rp, ci, B2d, C2, M, N, K, nnzb, plan=plan)
+    torch.cuda.synchronize()
+    plan.close()
+    edges = [g * 64 + d for g in range(8) for d in (0, 63)]
+    check_sampled(oracle, A, B, N, C.cpu().numpy().view(np.uint16), sample_rows(M // 16, 24, edges))
+    c, c2 = C.view(torch.float16), C2.view(torch.float16)
+    assert bool(torch.isfinite(c2).all()) and float(c.abs().max()) < 30000
+    tiny = c.abs() < 2.0**-13  # twice a subnormal result may round differently
+    assert bool(((c * 2 == c2) | tiny).all())
