@@ -154,6 +154,11 @@ __global__ __launch_bounds__(THREADS) void spmm_sweep_kernel(
 
     const int c_begin = rg_chunk_ptr[rg], n_chunks = rg_chunk_ptr[rg + 1] - c_begin;
     const int op_begin = op_ptr[rg * W + wave];
+    // the block rows this wavefront stores at the end (the plan spreads the rows of the group over the wavefronts):
+    // asked for here in two loads, so that the epilogue does not wait for eight of them one after the other
+    const i32x4 *my_rows = reinterpret_cast<const i32x4 *>(row_map + (rg * W + wave) * RW);
+    const i32x4 rows_lo = my_rows[0], rows_hi = my_rows[1];
+    static_assert(RW == 8, "two 16-byte loads hold the block rows of a wavefront");
 
     if (n_chunks > 0) { // uniform over the workgroup: every wavefront has the chunk list of its row group
         auto lds_copy = [&](uint32_t voff, const void *sbase, uint32_t dst) { // 64 lanes x 16 B -> LDS dst + lane * 16
@@ -222,7 +227,7 @@ __global__ __launch_bounds__(THREADS) void spmm_sweep_kernel(
     // Epilogue: tile (r, t), element e = C[(rg*64 + wave*8 + r)*16 + i16][n0 + 16*g + 4*t + e]
     auto store_row = [&](auto rc) {
         constexpr int R = decltype(rc)::value;
-        const int br = row_map[(rg * W + wave) * RW + R]; // the plan spreads the block rows of the group over the wavefronts
+        const int br = R < 4 ? rows_lo[R & 3] : rows_hi[R & 3];
         if (br < 0) return;
         const long m = (long)br * 16 + i16;
         const int nbase = n0 + 16 * g;
