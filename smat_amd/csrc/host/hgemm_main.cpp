@@ -5,7 +5,8 @@
 //   accepted and ignored: they only sized the dense-GEMM leftovers there)
 // and adds: -reorder (row + column clustering before blocking), -tau,
 //   -random_b (seeded uniform[-1,1] B instead of all ones), -use_plan, -kernel,
-//   -gpu_blocking (CSR -> BCSR on the device).  -filename also takes a binary container
+//   -gpu_blocking (CSR -> BCSR on the device), -poison_check (with -enable_check: plants one NaN in the result
+//   before it is compared, so the run must end with FAIL and a non-zero status).  -filename also takes a binary container
 //   written by smat_convert.  -lineplot [-lineplot_from=14 -lineplot_to=126 -lineplot_step=1] sweeps
 //   N = 8*mult like createLinePlot (common/tester.h:211-267) and appends "N, ms" lines to results_smat.csv.  Load, reorder and blocking times are logged apart from the SpMM time.
 #include <thread>
@@ -44,7 +45,8 @@ int main(int argc, char **argv)
                   (size_t)f.num("sleep_duration", 100), f.flag("enable_check", false),
                   lineplot ? lp_from + (lp_to - 1 - lp_from) / lp_step * lp_step : n_mult, file,
                   f.flag("reorder", false), (float)f.real("tau", 0.5), f.flag("random_b", false),
-                  f.flag("use_plan", true), (int)f.num("kernel", SMAT_KERNEL_AUTO), f.flag("gpu_blocking", false));
+                  f.flag("use_plan", true), (int)f.num("kernel", SMAT_KERNEL_AUTO), f.flag("gpu_blocking", false),
+                  f.flag("poison_check", false));
     if (lineplot) {
         if (!f.flag("use_plan", true)) { HLOG("-lineplot needs the plan (-use_plan)"); return 2; }
         tester.createLinePlot("Smat-Plan-Kernel", lp_from, lp_to, lp_step);

@@ -27,9 +27,9 @@ class Tester {
 public:
     Tester(size_t warmup_iterations, size_t profiling_iterations, size_t sleep_duration, bool enable_check,
            int n_mult, const std::string &filename, bool reorder, float tau, bool random_b, bool use_plan, int kernel,
-           bool gpu_blocking = false)
+           bool gpu_blocking = false, bool poison_check = false)
         : warmup_(warmup_iterations), iters_(profiling_iterations), sleep_ms_(sleep_duration), check_(enable_check),
-          file_(filename), kernel_(kernel)
+          poison_(poison_check), file_(filename), kernel_(kernel)
     {
         if (!warmup_ || !iters_) { HLOG("warmup_iterations and profiling_iterations must be positive"); exit(EXIT_FAILURE); }
         A_ = new SparseMatrix("Sparse Matrix A", filename, reorder, tau, gpu_blocking);
@@ -172,24 +172,34 @@ private:
         HLOG("CPU fp32 reference product: %.1f ms on 1 core", now_ms() - t0);
         C_->moveToHost();
         const size_t M = C_->getRow(), N = C_->getCol();
+        if (poison_) { // self-test of this check: one NaN in the copy of C that is looked at must fail the run
+            C_->getHostPtr()[(M / 2) * N + N / 2] = 0x7e00;
+            HLOG("-poison_check: one element of the result replaced by NaN before the comparison");
+        }
         double worst = 0, max_diff = 0, avg = 0;
+        size_t non_finite = 0;
         for (size_t i = 0; i < M; i++) {
             double nrm = 0, row_max = 0;
             for (size_t j = 0; j < N; j++) {
                 const double r = ref[i * N + j];
-                const double d = std::fabs((double)smat::half_to_float(C_->getHostPtr()[i * N + j]) - r);
+                double d = std::fabs((double)smat::half_to_float(C_->getHostPtr()[i * N + j]) - r);
+                if (!std::isfinite(d)) { // std::max would drop a NaN: a result that is not a number is a gross error
+                    d = 1e30;
+                    non_finite++;
+                }
                 nrm += r * r; row_max = std::max(row_max, d); avg += d;
             }
             max_diff = std::max(max_diff, row_max);
             worst = std::max(worst, nrm > 0 ? row_max / std::sqrt(nrm) : row_max);
         }
         HLOG("Max diff: %f, avg diff: %f", max_diff, avg / (double)(M * N));
+        if (non_finite) HLOG("%zu elements of the result are not finite where the reference product is", non_finite);
         HLOG("Max error relative to the row L2 norm: %.3e (%s, bound 1e-3)", worst, worst <= 1e-3 ? "PASS" : "FAIL");
         if (!(worst <= 1e-3)) exit(EXIT_FAILURE);
     }
 
     size_t warmup_, iters_, sleep_ms_;
-    bool check_;
+    bool check_, poison_;
     std::string file_;
     int kernel_;
     SparseMatrix *A_ = nullptr;

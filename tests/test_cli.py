@@ -108,3 +108,17 @@ def test_hgemm_lineplot_sweeps_n(tmp_path):
     lines = (tmp_path / "results_smat.csv").read_text().strip().splitlines()
     assert [int(ln.split(",")[0]) for ln in lines] == [112, 152, 192, 232]
     assert all(float(ln.split(",")[1]) > 0 for ln in lines)
+
+
+@pytest.mark.gpu
+def test_hgemm_check_fails_on_a_nan_in_the_result(tmp_path):
+    """The verify step treats a result that is not a number as a gross error: one NaN planted in C ends the run with
+    FAIL and a non-zero status (a maximum taken with std::max alone would never see it)."""
+    d = gen.stencil27(10)
+    mtx = tmp_path / "stencil10.mtx"
+    write_mtx(mtx, d)
+    cmd = [os.path.join(BIN, "hgemm"), f"-filename={mtx}", "-n_mult=9", "-enable_check", "-random_b",
+           "-warmup_iterations=1", "-profiling_iterations=1", "-sleep_duration=1", "-poison_check"]
+    run = subprocess.run(cmd, cwd=tmp_path, capture_output=True, text=True, timeout=120)
+    assert run.returncode != 0
+    assert "FAIL" in run.stderr and "PASS" not in run.stderr and "not finite" in run.stderr
