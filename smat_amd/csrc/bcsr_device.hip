@@ -21,6 +21,7 @@
 #include <stdint.h>
 
 #include "../../include/smat.h"
+#include "devmem.h"
 #include "errors.h"
 
 using namespace smat;
@@ -147,8 +148,8 @@ __global__ void count_flags_kernel(const uint8_t *__restrict__ flags, int64_t n,
 
 struct Scratch {
     void *p = nullptr;
-    ~Scratch() { if (p) (void)hipFree(p); }
-    hipError_t alloc(size_t bytes) { return hipMalloc(&p, bytes ? bytes : 16); }
+    ~Scratch() { if (p) (void)dev_free(p); }
+    hipError_t alloc(size_t bytes) { return dev_malloc(&p, bytes ? bytes : 16); }
 };
 
 } // namespace
@@ -209,9 +210,9 @@ static int smat_csr_to_bcsr_device_impl(size_t M, size_t K, const int32_t *row_p
 
     int32_t *orp = nullptr, *oci = nullptr;
     uint16_t *ov = nullptr;
-    hipError_t e = hipMalloc(&orp, (mb + 1) * sizeof(int32_t));
-    if (e == hipSuccess) e = hipMalloc(&oci, std::max<size_t>(nnzb, 1) * sizeof(int32_t));
-    if (e == hipSuccess) e = hipMalloc(&ov, std::max<size_t>(nnzb, 1) * 512);
+    hipError_t e = dev_malloc(&orp, (mb + 1) * sizeof(int32_t));
+    if (e == hipSuccess) e = dev_malloc(&oci, std::max<size_t>(nnzb, 1) * sizeof(int32_t));
+    if (e == hipSuccess) e = dev_malloc(&ov, std::max<size_t>(nnzb, 1) * 512);
     if (e == hipSuccess) e = hipMemset(ov, 0, std::max<size_t>(nnzb, 1) * 512);
     if (e == hipSuccess) e = flags.alloc(std::max<size_t>(nnzb, 1));
     if (e == hipSuccess) e = hipMemset(flags.p, 0, std::max<size_t>(nnzb, 1));
@@ -247,9 +248,9 @@ static int smat_csr_to_bcsr_device_impl(size_t M, size_t K, const int32_t *row_p
     }
     if (e == hipSuccess) e = hipDeviceSynchronize();
     if (e != hipSuccess) {
-        if (orp) (void)hipFree(orp);
-        if (oci) (void)hipFree(oci);
-        if (ov) (void)hipFree(ov);
+        if (orp) (void)dev_free(orp);
+        if (oci) (void)dev_free(oci);
+        if (ov) (void)dev_free(ov);
         return set_error(SMAT_ERR_HIP, "device blocking failed: %s", hipGetErrorString(e));
     }
     if (counts) {

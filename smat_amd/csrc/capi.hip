@@ -11,6 +11,7 @@
 #include <vector>
 
 #include "../../include/smat.h"
+#include "devmem.h"
 #include "errors.h"
 #include "spmm_kernels.h"
 #include "sweep_plan.h"
@@ -78,7 +79,7 @@ hipError_t smat_plan::SweepDev::upload(const SweepPlanHost &h)
     hipError_t e = hipSuccess;
     auto up = [&](void **dst, const void *src, size_t bytes) {
         if (e != hipSuccess) return;
-        e = hipMalloc(dst, std::max<size_t>(bytes, 16));
+        e = dev_malloc(dst, std::max<size_t>(bytes, 16));
         if (e == hipSuccess && bytes) e = hipMemcpy(*dst, src, bytes, hipMemcpyHostToDevice);
     };
     up((void **)&d_rg_chunk_ptr, h.rg_chunk_ptr.data(), h.rg_chunk_ptr.size() * sizeof(int32_t));
@@ -92,10 +93,20 @@ hipError_t smat_plan::SweepDev::upload(const SweepPlanHost &h)
 void smat_plan::SweepDev::release()
 {
     for (void *q : {(void *)d_rg_chunk_ptr, (void *)d_chunk_ids, (void *)d_op_ptr, (void *)d_row_map, (void *)d_ops})
-        if (q) (void)hipFree(q);
+        if (q) (void)dev_free(q);
     d_rg_chunk_ptr = d_chunk_ids = d_op_ptr = d_row_map = nullptr;
     d_ops = nullptr;
     n_rg = n_records = n_ops = 0;
+}
+
+namespace smat {
+std::atomic<long long> g_dev_mallocs{0}, g_dev_frees{0};
+}
+// Test hook (not part of smat.h): device allocations and releases made by the library since it was loaded.
+extern "C" void smat_internal_alloc_counts(int64_t *out)
+{
+    out[0] = g_dev_mallocs.load();
+    out[1] = g_dev_frees.load();
 }
 
 extern "C" const char *smat_version(void) { return "smat-amd 0.1 gfx950"; }
@@ -396,15 +407,15 @@ static int smat_plan_create_impl(smat_plan **out, const int32_t *row_ptr_host,
     p->n_split_rows = (int)split.size();
     p->n_slots = slot;
 
-    hipError_t e = hipMalloc(&p->d_items, std::max<size_t>(items.size(), 1) * sizeof(WorkItem));
+    hipError_t e = dev_malloc(&p->d_items, std::max<size_t>(items.size(), 1) * sizeof(WorkItem));
     if (e == hipSuccess && !items.empty())
         e = hipMemcpy(p->d_items, items.data(), items.size() * sizeof(WorkItem), hipMemcpyHostToDevice);
     if (e == hipSuccess && !split.empty()) {
-        e = hipMalloc(&p->d_split, split.size() * sizeof(SplitRow));
+        e = dev_malloc(&p->d_split, split.size() * sizeof(SplitRow));
         if (e == hipSuccess)
             e = hipMemcpy(p->d_split, split.data(), split.size() * sizeof(SplitRow), hipMemcpyHostToDevice);
         p->workspace_bytes = (size_t)slot * 16 * n_hint * sizeof(float);
-        if (e == hipSuccess) e = hipMalloc(&p->d_workspace, p->workspace_bytes);
+        if (e == hipSuccess) e = dev_malloc(&p->d_workspace, p->workspace_bytes);
     }
     // Row-wise kernel: repacking B slab-major costs a launch plus one read and one write of B
     // per SpMM (about 3 us + 4*K*N bytes at 4 TB/s) and lets the operand gather, nnzb*16*N*2
@@ -415,7 +426,7 @@ static int smat_plan_create_impl(smat_plan **out, const int32_t *row_ptr_host,
         const double cost_us = 3.0 + 4.0 * (double)K * (double)n_hint / 4e6;
         if (e == hipSuccess && want != SMAT_KERNEL_ROWWISE_DIRECT &&
             (gain_us > 1.5 * cost_us || want == SMAT_KERNEL_ROWWISE_PACKED))
-            e = hipMalloc(&p->d_bpack, K * n_hint * sizeof(uint16_t));
+            e = dev_malloc(&p->d_bpack, K * n_hint * sizeof(uint16_t));
     }
     // The sweep kernel pays one pass over the B panel per group of 32 block rows,
     // whatever the sparsity, and shares each staged slab between the blocks of the group
@@ -423,7 +434,7 @@ static int smat_plan_create_impl(smat_plan **out, const int32_t *row_ptr_host,
     // M = K in {4096, 8192, 16384}, N in {512 .. 4096} and 5% .. 25% of the blocks present: it
     // wins (by 1.02x at 5% up to 1.6x at 25%) whenever its workgroups (groups of 32 block
     // rows x panels of 128 columns) fill the 256 CUs, and loses (0.3x .. 0.9x) when they do not.
-    if (e == hipSuccess && opts && opts->b_layout == SMAT_B_ROW_MAJOR) e = hipMalloc(&p->d_bcol, K * n_hint * sizeof(uint16_t));
+    if (e == hipSuccess && opts && opts->b_layout == SMAT_B_ROW_MAJOR) e = dev_malloc(&p->d_bcol, K * n_hint * sizeof(uint16_t));
     bool sweep = want == SMAT_KERNEL_SWEEP;
     if (want == SMAT_KERNEL_AUTO && col_idx_host && sweep_fills_device(mb, n_hint) &&
         (double)nnzb >= 0.05 * (double)mb * (double)kb)
@@ -440,7 +451,7 @@ static int smat_plan_create_impl(smat_plan **out, const int32_t *row_ptr_host,
         static_assert(sizeof(SweepOpHost) == sizeof(SweepOp), "host and device op layouts");
         e = p->sweep.upload(h);
         if (p->d_bpack && want != SMAT_KERNEL_ROWWISE_PACKED) { // the sweep kernel reads B in place
-            (void)hipFree(p->d_bpack);
+            (void)dev_free(p->d_bpack);
             p->d_bpack = nullptr;
         }
     }
@@ -470,9 +481,9 @@ static int smat_plan_attach_values_impl(smat_plan *p, const uint16_t *vals, cons
     const int dense_kernel = p->sweep.d_ops ? SMAT_KERNEL_SWEEP : SMAT_KERNEL_ROWWISE;
     auto drop_mixed = [&] {
         p->sweep_dense.release();
-        if (p->d_items_dense) { (void)hipFree(p->d_items_dense); p->d_items_dense = nullptr; }
-        if (p->d_split_dense) { (void)hipFree(p->d_split_dense); p->d_split_dense = nullptr; }
-        if (p->d_workspace_dense) { (void)hipFree(p->d_workspace_dense); p->d_workspace_dense = nullptr; }
+        if (p->d_items_dense) { (void)dev_free(p->d_items_dense); p->d_items_dense = nullptr; }
+        if (p->d_split_dense) { (void)dev_free(p->d_split_dense); p->d_split_dense = nullptr; }
+        if (p->d_workspace_dense) { (void)dev_free(p->d_workspace_dense); p->d_workspace_dense = nullptr; }
         p->n_items_dense = p->n_split_dense = 0;
         p->n_blocks_dense = 0;
     };
@@ -514,7 +525,7 @@ static int smat_plan_attach_values_impl(smat_plan *p, const uint16_t *vals, cons
         if (p->kernel == SMAT_KERNEL_COMPACT || p->kernel == SMAT_KERNEL_MIXED) p->kernel = dense_kernel;
         return SMAT_OK;
     }
-    if (!p->d_bt) e = hipMalloc(&p->d_bt, p->bt_bytes());
+    if (!p->d_bt) e = dev_malloc(&p->d_bt, p->bt_bytes());
     // the dense rows through the sweep kernel when their row groups of 64 fill the device, else row-wise
     std::vector<int32_t> dense_list;
     for (size_t i = 0; mixed && i < mb; i++)
@@ -533,13 +544,13 @@ static int smat_plan_attach_values_impl(smat_plan *p, const uint16_t *vals, cons
         p->n_items_dense = (int)items.size();
         p->n_split_dense = (int)split.size();
         p->n_blocks_dense = blocks_dense;
-        e = hipMalloc(&p->d_items_dense, std::max<size_t>(items.size(), 1) * sizeof(WorkItem));
+        e = dev_malloc(&p->d_items_dense, std::max<size_t>(items.size(), 1) * sizeof(WorkItem));
         if (e == hipSuccess && !items.empty())
             e = hipMemcpy(p->d_items_dense, items.data(), items.size() * sizeof(WorkItem), hipMemcpyHostToDevice);
         if (e == hipSuccess && !split.empty()) {
-            e = hipMalloc(&p->d_split_dense, split.size() * sizeof(SplitRow));
+            e = dev_malloc(&p->d_split_dense, split.size() * sizeof(SplitRow));
             if (e == hipSuccess) e = hipMemcpy(p->d_split_dense, split.data(), split.size() * sizeof(SplitRow), hipMemcpyHostToDevice);
-            if (e == hipSuccess) e = hipMalloc(&p->d_workspace_dense, (size_t)slots * 16 * p->n_cap * sizeof(float));
+            if (e == hipSuccess) e = dev_malloc(&p->d_workspace_dense, (size_t)slots * 16 * p->n_cap * sizeof(float));
         }
     }
     if (e != hipSuccess) {
@@ -549,7 +560,7 @@ static int smat_plan_attach_values_impl(smat_plan *p, const uint16_t *vals, cons
     p->compact = c;
     p->kernel = mixed ? SMAT_KERNEL_MIXED : SMAT_KERNEL_COMPACT;
     if (p->d_bpack && want == SMAT_KERNEL_AUTO && !mixed) { // the row-wise kernel's scratch is not needed any more
-        (void)hipFree(p->d_bpack);
+        (void)dev_free(p->d_bpack);
         p->d_bpack = nullptr;
     }
     return SMAT_OK;
@@ -565,15 +576,15 @@ extern "C" int smat_plan_destroy(smat_plan *p)
 {
     if (!p) return SMAT_OK;
     if (p->compact) compact_destroy(p->compact);
-    if (p->d_bt) (void)hipFree(p->d_bt);
-    if (p->d_bcol) (void)hipFree(p->d_bcol);
-    if (p->d_items_dense) (void)hipFree(p->d_items_dense);
-    if (p->d_split_dense) (void)hipFree(p->d_split_dense);
-    if (p->d_workspace_dense) (void)hipFree(p->d_workspace_dense);
-    if (p->d_items) (void)hipFree(p->d_items);
-    if (p->d_split) (void)hipFree(p->d_split);
-    if (p->d_workspace) (void)hipFree(p->d_workspace);
-    if (p->d_bpack) (void)hipFree(p->d_bpack);
+    if (p->d_bt) (void)dev_free(p->d_bt);
+    if (p->d_bcol) (void)dev_free(p->d_bcol);
+    if (p->d_items_dense) (void)dev_free(p->d_items_dense);
+    if (p->d_split_dense) (void)dev_free(p->d_split_dense);
+    if (p->d_workspace_dense) (void)dev_free(p->d_workspace_dense);
+    if (p->d_items) (void)dev_free(p->d_items);
+    if (p->d_split) (void)dev_free(p->d_split);
+    if (p->d_workspace) (void)dev_free(p->d_workspace);
+    if (p->d_bpack) (void)dev_free(p->d_bpack);
     p->sweep.release();
     p->sweep_dense.release();
     delete p;
@@ -653,10 +664,10 @@ extern "C" int smat_device_attr(int dev, int64_t *cus, int64_t *lds_bytes, int64
 extern "C" int smat_malloc(void **dptr, size_t bytes)
 {
     if (!dptr) return set_error(SMAT_ERR_INVALID, "dptr must not be NULL");
-    SMAT_HIP(hipMalloc(dptr, bytes ? bytes : 1));
+    SMAT_HIP(dev_malloc(dptr, bytes ? bytes : 1));
     return SMAT_OK;
 }
-extern "C" int smat_free(void *dptr) { if (dptr) SMAT_HIP(hipFree(dptr)); return SMAT_OK; }
+extern "C" int smat_free(void *dptr) { if (dptr) SMAT_HIP(dev_free(dptr)); return SMAT_OK; }
 extern "C" int smat_memcpy_h2d(void *d, const void *s, size_t n) { if (n) SMAT_HIP(hipMemcpy(d, s, n, hipMemcpyHostToDevice)); return SMAT_OK; }
 extern "C" int smat_memcpy_d2h(void *d, const void *s, size_t n) { if (n) SMAT_HIP(hipMemcpy(d, s, n, hipMemcpyDeviceToHost)); return SMAT_OK; }
 extern "C" int smat_memcpy_d2d(void *d, const void *s, size_t n) { if (n) SMAT_HIP(hipMemcpy(d, s, n, hipMemcpyDeviceToDevice)); return SMAT_OK; }
@@ -724,7 +735,7 @@ extern "C" int smat_bench_mfma_peak(double *tflops)
     SMAT_HIP(hipGetDeviceProperties(&prop, dev));
     const int cus = prop.multiProcessorCount, iters = 16384;
     float *out = nullptr;
-    SMAT_HIP(hipMalloc(&out, sizeof(float)));
+    SMAT_HIP(dev_malloc(&out, sizeof(float)));
     hipEvent_t e0, e1;
     SMAT_HIP(hipEventCreate(&e0));
     SMAT_HIP(hipEventCreate(&e1));
@@ -741,7 +752,7 @@ extern "C" int smat_bench_mfma_peak(double *tflops)
     }
     (void)hipEventDestroy(e0);
     (void)hipEventDestroy(e1);
-    (void)hipFree(out);
+    (void)dev_free(out);
     SMAT_HIP(hipGetLastError());
     *tflops = best;
     return SMAT_OK;

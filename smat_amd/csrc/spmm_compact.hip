@@ -40,6 +40,7 @@
 #include <algorithm>
 #include <vector>
 
+#include "devmem.h"
 #include "spmm_kernels.h"
 
 namespace smat {
@@ -353,8 +354,8 @@ hipError_t launch_compact_tq(const CompactArgs &a, hipStream_t st)
 
 struct Scratch {
     void *p = nullptr;
-    ~Scratch() { if (p) (void)hipFree(p); }
-    hipError_t alloc(size_t bytes) { return hipMalloc(&p, bytes ? bytes : 16); }
+    ~Scratch() { if (p) (void)dev_free(p); }
+    hipError_t alloc(size_t bytes) { return dev_malloc(&p, bytes ? bytes : 16); }
 };
 
 } // namespace
@@ -401,7 +402,7 @@ hipError_t values_checksum(const uint16_t *vals, size_t nnzb, uint64_t *out)
     *out = 0;
     if (!nnzb) return hipSuccess;
     unsigned long long *d = nullptr;
-    hipError_t e = hipMalloc(&d, sizeof(unsigned long long));
+    hipError_t e = dev_malloc(&d, sizeof(unsigned long long));
     if (e != hipSuccess) return e;
     e = hipMemset(d, 0, sizeof(unsigned long long));
     if (e == hipSuccess) {
@@ -412,7 +413,7 @@ hipError_t values_checksum(const uint16_t *vals, size_t nnzb, uint64_t *out)
     }
     unsigned long long h = 0;
     if (e == hipSuccess) e = hipMemcpy(&h, d, sizeof h, hipMemcpyDeviceToHost);
-    (void)hipFree(d);
+    (void)dev_free(d);
     *out = h;
     return e;
 }
@@ -420,11 +421,11 @@ hipError_t values_checksum(const uint16_t *vals, size_t nnzb, uint64_t *out)
 void compact_destroy(CompactPlan *p)
 {
     if (!p) return;
-    if (p->d_cols) (void)hipFree(p->d_cols);
-    if (p->d_acol) (void)hipFree(p->d_acol);
-    if (p->d_items) (void)hipFree(p->d_items);
-    if (p->d_split) (void)hipFree(p->d_split);
-    if (p->d_workspace) (void)hipFree(p->d_workspace);
+    if (p->d_cols) (void)dev_free(p->d_cols);
+    if (p->d_acol) (void)dev_free(p->d_acol);
+    if (p->d_items) (void)dev_free(p->d_items);
+    if (p->d_split) (void)dev_free(p->d_split);
+    if (p->d_workspace) (void)dev_free(p->d_workspace);
     delete p;
 }
 
@@ -489,9 +490,9 @@ hipError_t compact_build(const uint16_t *vals, const int32_t *row_ptr, const int
     padded[mb] = (int32_t)total;
     padded_dev[mb] = (int32_t)total;
     const size_t cap = (size_t)total + LIST_PAD;
-    SMAT_STEP(hipMalloc(&p->d_cols, cap * sizeof(int32_t)));
+    SMAT_STEP(dev_malloc(&p->d_cols, cap * sizeof(int32_t)));
     SMAT_STEP(hipMemset(p->d_cols, 0, cap * sizeof(int32_t))); // padding: row 0 of B
-    SMAT_STEP(hipMalloc(&p->d_acol, cap * 16 * sizeof(uint16_t)));
+    SMAT_STEP(dev_malloc(&p->d_acol, cap * 16 * sizeof(uint16_t)));
     SMAT_STEP(hipMemset(p->d_acol, 0, cap * 16 * sizeof(uint16_t)));
     if (e == hipSuccess && nnzb) {
         SMAT_STEP(hipMemcpy(cc.p, padded_dev.data(), (mb + 1) * 4, hipMemcpyHostToDevice));
@@ -531,12 +532,12 @@ hipError_t compact_build(const uint16_t *vals, const int32_t *row_ptr, const int
     p->n_items = (int)items.size();
     p->n_split_rows = (int)split.size();
     p->n_slots = slot;
-    SMAT_STEP(hipMalloc(&p->d_items, std::max<size_t>(items.size(), 1) * sizeof(WorkItem)));
+    SMAT_STEP(dev_malloc(&p->d_items, std::max<size_t>(items.size(), 1) * sizeof(WorkItem)));
     if (!items.empty()) SMAT_STEP(hipMemcpy(p->d_items, items.data(), items.size() * sizeof(WorkItem), hipMemcpyHostToDevice));
     if (!split.empty()) {
-        SMAT_STEP(hipMalloc(&p->d_split, split.size() * sizeof(SplitRow)));
+        SMAT_STEP(dev_malloc(&p->d_split, split.size() * sizeof(SplitRow)));
         SMAT_STEP(hipMemcpy(p->d_split, split.data(), split.size() * sizeof(SplitRow), hipMemcpyHostToDevice));
-        SMAT_STEP(hipMalloc(&p->d_workspace, (size_t)slot * 16 * n_cap * sizeof(float)));
+        SMAT_STEP(dev_malloc(&p->d_workspace, (size_t)slot * 16 * n_cap * sizeof(float)));
     }
     SMAT_STEP(values_checksum(vals, nnzb, &p->values_checksum));
     SMAT_STEP(hipDeviceSynchronize());

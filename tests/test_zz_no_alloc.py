@@ -17,6 +17,13 @@ def to_dev(torch, a, cuda):
     return torch.from_numpy(np.ascontiguousarray(a).view(np.int16) if a.dtype == np.uint16 else np.ascontiguousarray(a)).to(cuda)
 
 
+def alloc_counts():
+    from smat_amd._lib import lib
+    out = (C.c_int64 * 2)()
+    lib.smat_internal_alloc_counts(out)
+    return out[0], out[1]
+
+
 def run_both(smat, cuda, A, B_bits, N):
     import torch
     from smat_amd._lib import lib, check
@@ -24,19 +31,27 @@ def run_both(smat, cuda, A, B_bits, N):
     vals, Bd = to_dev(torch, A["b_val"], cuda), to_dev(torch, B_bits, cuda)
     rp, ci = to_dev(torch, A["b_row_ptr"].astype(np.int32), cuda), to_dev(torch, A["b_col_idx"].astype(np.int32), cuda)
     # existing entry point: plan-owned copy of B
+    counts_before_plan = alloc_counts()
     C_ref = torch.full((M, N), 0x7E00, dtype=torch.int16, device=cuda)
     plan = smat.Plan(A["b_row_ptr"], M, K, nnzb, N, col_idx_host=A["b_col_idx"], kernel=ROWWISE_PACKED)
     assert plan.info()["split_rows"] == 0 and plan.info()["b_pack_bytes"] == K * N * 2
     smat.spmm(vals, rp, ci, Bd, C_ref, M, N, K, nnzb, plan=plan, kernel=ROWWISE_PACKED)
     torch.cuda.synchronize()
     plan.close()
-    # the entry point under test: no plan, no allocation
+    # the entry point under test: no plan, no allocation.  Witnesses: the library's own count of its device
+    # allocations and releases (every one of them goes through the counted wrappers of devmem.h), and the free
+    # device memory the driver reports (which a hipMalloc inside the library would lower, whoever made it).
     C_new = torch.full((M, N), 0x7E00, dtype=torch.int16, device=cuda)
-    before = torch.cuda.memory_allocated()
-    check(lib.smat_spmm_bcsr_f16_static(vals.data_ptr(), rp.data_ptr(), ci.data_ptr(), Bd.data_ptr(), C_new.data_ptr(),
-                                        M, N, K, nnzb, None))
     torch.cuda.synchronize()
-    assert torch.cuda.memory_allocated() == before
+    after_plan = alloc_counts()
+    assert after_plan[0] > counts_before_plan[0], "the counters do not see the plan's allocations"
+    free_before = torch.cuda.mem_get_info()[0]
+    for _ in range(3):
+        check(lib.smat_spmm_bcsr_f16_static(vals.data_ptr(), rp.data_ptr(), ci.data_ptr(), Bd.data_ptr(), C_new.data_ptr(),
+                                            M, N, K, nnzb, None))
+    torch.cuda.synchronize()
+    assert alloc_counts() == after_plan, "smat_spmm_bcsr_f16_static allocated or released device memory"
+    assert torch.cuda.mem_get_info()[0] >= free_before
     return C_ref.cpu().numpy().view(np.uint16), C_new.cpu().numpy().view(np.uint16)
 
 
