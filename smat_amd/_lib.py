@@ -6,8 +6,8 @@ _HERE = os.path.dirname(os.path.abspath(__file__))
 
 
 def library_path():
-    """In-tree library; SMAT_AMD_LIBRARY overrides it (to try an experimental build)."""
-    return os.environ.get("SMAT_AMD_LIBRARY") or os.path.join(_HERE, "libsmat_amd.so")
+    """The in-tree library."""
+    return os.path.join(_HERE, "libsmat_amd.so")
 
 
 class SmatError(RuntimeError):

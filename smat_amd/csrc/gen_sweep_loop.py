@@ -16,7 +16,7 @@ Run after changing:
 
     python3 gen_sweep_loop.py > spmm_sweep_loop.inc
 
-Stream position i, J = i % 8.  Block of op i (default: --lds-ahead 1 --ahead 4):
+Stream position i, J = i % 8.  Block of op i (AHEAD = 4):
     even position: LDS reads of the B operands of op i + 1 (into set (J + 1) % 2), then a wait until only those
     four are left: LDS reads return in order, so the reads of op i are in registers.  Scalar loads share the
     counter and return in any order; with one of them under way the same wait holds for the reads of op i
@@ -28,12 +28,10 @@ Stream position i, J = i % 8.  Block of op i (default: --lds-ahead 1 --ahead 4):
     The set that the reads of op i + 1 land in is the one the MFMAs of op i - 1 took their operands from a few
     instructions earlier: an MFMA reads its A and B sources when it starts, LDS data arrives 64 clocks later
     at the earliest.
-With --lds-ahead 2 every position issues the reads of op i + 2 (four sets), odd positions load the descriptors of
-ops i + 5 and i + 6, and the A ring has four slots (--ahead 2 or 3): the earlier pipeline, kept for comparison.
 Marker (first thing of every chunk but the first): own copies of the next chunk have landed, barrier,
 copies of the chunk after next, and the same read-ahead duties, no MFMAs.
 
-Registers (fixed, all listed as clobbers; --lds-ahead 1):
+Registers (fixed, all listed as clobbers):
     v40-v71    B operands, two sets of 4 tiles x 4 registers
     v72-v103   A operands, ring of eight
     v104-v106  temporaries
@@ -43,23 +41,16 @@ Registers (fixed, all listed as clobbers; --lds-ahead 1):
     a0-a127    accumulators (block row r, tile t in a[16r + 4t .. + 3])
 """
 
-import argparse
+import sys
 
-ap = argparse.ArgumentParser()
-ap.add_argument("--ahead", type=int, default=4, help="A operands are loaded this many ops ahead (2..5 with --lds-ahead 1: ring of eight; 2..3 with --lds-ahead 2: ring of four)")
-ap.add_argument("--lds-ahead", type=int, default=1, help="B operands are read from LDS this many positions ahead: 2 (four register sets, A ring of four) or 1 (two sets, A ring of eight, --ahead up to 5)")
-ap.add_argument("--block-bytes", type=int, default=128, help="size of an op block's slot (SWEEP_BLOCK_BYTES)")
-ap.add_argument("--ablate", default="", help="timing experiments only, wrong results: any of a,copy,barrier,mfma,bread,vm")
-args = ap.parse_args()
-AHEAD = args.ahead
-LB = args.lds_ahead
-ABL = set(x for x in args.ablate.split(",") if x)
-assert LB in (1, 2)
-BSETS, ARING = (4, 4) if LB == 2 else (2, 8)
-assert 2 <= AHEAD <= (3 if LB == 2 else 5)
+if len(sys.argv) > 1:
+    sys.exit("gen_sweep_loop.py takes no arguments: it writes the one loop the library ships")
+
+AHEAD = 4                                # SWEEP_AHEAD: A operands are loaded this many stream positions ahead (ring of eight)
+BSETS, ARING = 2, 8                      # B operands are read from LDS one position ahead (two register sets)
 
 RING = 8
-BLOCK_BYTES = args.block_bytes           # SWEEP_BLOCK_BYTES
+BLOCK_BYTES = 128                        # SWEEP_BLOCK_BYTES
 MARK_BASE = 8 * 8 * 2 * BLOCK_BYTES      # SWEEP_MARK_BASE: after the 128 op blocks
 MARK_BYTES = 512                         # SWEEP_MARK_BYTES
 END_OFF = MARK_BASE + 8 * MARK_BYTES     # SWEEP_END_OFF
@@ -68,7 +59,7 @@ MIN_OPS = max(AHEAD - 1, COPIES)
 VM_MARK = MIN_OPS + 1      # a marker's copies of one marker ago are older than the A loads of the MIN_OPS + 1 positions since
 
 S_RING0 = 40
-DESC_AHEAD = 5 if LB == 2 else 7   # an odd position loads the descriptors of ops i + DESC_AHEAD and the one after
+DESC_AHEAD = 7   # an odd position loads the descriptors of ops i + DESC_AHEAD and the one after
 S_DP, S_BASE, S_CUR, S_NEXTK, S_CP, S_T0, S_T1, S_JMP = 72, 74, 76, 77, 78, 80, 81, 84
 S_LAST = 85
 V_B0 = 40
@@ -109,42 +100,27 @@ def b_reads(dst_set, desc_slot):
     emit(f"v_xad_u32 v{V_T1}, v{V_T0}, %[lane_xor], %[rd_lane]")
     for t in range(4):
         off = f" offset:{1024 * t}" if t else ""
-        if "bread" in ABL:
-            continue
         emit(f"ds_read_b128 {bset(dst_set, t)}, v{V_T1}{off}")
 
 
 def a_load(slot):
-    if "a" in ABL:
-        return
     emit(f"buffer_load_dwordx4 {aslot(slot)}, %[a_voff], %[rsrc], {ring(slot, 0)} offen")
 
 
 def top_wait(J):
-    """B operands of op i are in registers.  Odd positions: everything asked for so far is, and the next two descriptors are asked for."""
-    if LB == 1:
-        # reads one position ahead: an even position asks for those of op i + 1 first and waits until only they are
-        # left; an odd position waits for everything (reads of op i, descriptors asked for two positions ago),
-        # asks for two descriptors and then for the reads of op i + 1
-        if J % 2 == 0:
-            b_reads(J + 1, J + 1)
-            emit("s_waitcnt lgkmcnt(4)")
-            return
-        emit("s_waitcnt lgkmcnt(0)")
-        s0 = S_RING0 + 4 * ((J + DESC_AHEAD) % RING)
-        emit(f"s_load_dwordx8 s[{s0}:{s0 + 7}], s[{S_DP}:{S_DP + 1}], 0x0")
-        emit(f"s_add_u32 s{S_DP}, s{S_DP}, 32")
-        emit(f"s_addc_u32 s{S_DP + 1}, s{S_DP + 1}, 0")
-        b_reads(J + 1, J + 1)
-        return
+    """B operands of op i are in registers.  An even position asks for the reads of op i + 1 first and waits until
+    only they are left; an odd position waits for everything (reads of op i, descriptors asked for two positions
+    ago), asks for two descriptors and then for the reads of op i + 1."""
     if J % 2 == 0:
+        b_reads(J + 1, J + 1)
         emit("s_waitcnt lgkmcnt(4)")
         return
     emit("s_waitcnt lgkmcnt(0)")
-    s0 = S_RING0 + 4 * ((J + 5) % RING)                # ops i + 5, i + 6: slots free since ops i - 3, i - 2
+    s0 = S_RING0 + 4 * ((J + DESC_AHEAD) % RING)
     emit(f"s_load_dwordx8 s[{s0}:{s0 + 7}], s[{S_DP}:{S_DP + 1}], 0x0")
     emit(f"s_add_u32 s{S_DP}, s{S_DP}, 32")
     emit(f"s_addc_u32 s{S_DP + 1}, s{S_DP + 1}, 0")
+    b_reads(J + 1, J + 1)
 
 
 def jump(desc_slot):
@@ -157,25 +133,10 @@ def op_block(J, r, v):
     k = (J * 8 + r) * 2 + v
     label(f"Lb{k}")
     top_wait(J)
-    if LB == 2:
-        b_reads(J + 2, J + 2)
     a_load(J + AHEAD)
-    for x in ABL:   # experiments on instruction fetch: padlit4 = 4 scalar moves with a literal (32 bytes), pad4 / pad8 = without (16 / 32 bytes)
-        if x.startswith("padlit"):
-            for _ in range(int(x[6:])):
-                emit("s_mov_b32 s86, 0x12345678")
-        elif x.startswith("pad"):
-            for _ in range(int(x[3:])):
-                emit("s_mov_b32 s86, 1")
-    if "vm" not in ABL:
-        emit(f"s_waitcnt vmcnt({AHEAD + COPIES * v})")
+    emit(f"s_waitcnt vmcnt({AHEAD + COPIES * v})")
     for t in range(4):
         acc = f"a[{16 * r + 4 * t}:{16 * r + 4 * t + 3}]"
-        if "mfma" in ABL:
-            continue
-        if "swap" in ABL:
-            emit(f"v_mfma_f32_16x16x32_f16 {acc}, {aslot(J)}, {bset(J, t)}, {acc}")
-            continue
         emit(f"v_mfma_f32_16x16x32_f16 {acc}, {bset(J, t)}, {aslot(J)}, {acc}")
     jump(J + 1)
     emit(f".org Lb0_%= + {(k + 1) * BLOCK_BYTES}")
@@ -185,8 +146,7 @@ def marker_block(J):
     label(f"Lm{J}")
     top_wait(J)                                       # the reads of the ops of the chunk that ends here are in registers
     emit(f"s_waitcnt vmcnt({VM_MARK})")               # own copies of the chunk after the one being entered (issued one marker ago) have landed
-    if "barrier" not in ABL:
-        emit("s_barrier")
+    emit("s_barrier")
     emit(f"s_add_u32 s{S_CUR}, s{S_CUR}, 1")          # chunk (position in the row group's list) being entered
     emit(f"s_add_u32 s{S_T0}, s{S_CUR}, 2")
     emit(f"s_cmp_ge_u32 s{S_T0}, %[n_chunks]")
@@ -201,14 +161,11 @@ def marker_block(J):
     for it in range(COPIES):
         emit(f"s_add_u32 m0, s{S_T0}, {1024 * it}")
         emit("s_nop 0")
-        if "copy" not in ABL:
-            emit(f"global_load_lds_dwordx4 v{V_COPY}, %[sb{it}]")
+        emit(f"global_load_lds_dwordx4 v{V_COPY}, %[sb{it}]")
     label(f"Lmn{J}")
     emit(f"s_load_dword s{S_NEXTK}, s[{S_CP}:{S_CP + 1}], 0x0")   # id of chunk cur + 3, for the next marker
     emit(f"s_add_u32 s{S_CP}, s{S_CP}, 4")
     emit(f"s_addc_u32 s{S_CP + 1}, s{S_CP + 1}, 0")
-    if LB == 2:
-        b_reads(J + 2, J + 2)
     a_load(J + AHEAD)
     jump(J + 1)
     emit(f".org Lb0_%= + {MARK_BASE + (J + 1) * MARK_BYTES}")
@@ -218,11 +175,8 @@ def marker_block(J):
 emit(f"s_mov_b32 s{S_DP}, %[op_lo]")
 emit(f"s_mov_b32 s{S_DP + 1}, %[op_hi]")
 emit(f"s_load_dwordx16 s[{S_RING0}:{S_RING0 + 15}], s[{S_DP}:{S_DP + 1}], 0x0")
-if LB == 2:
-    emit(f"s_load_dwordx8 s[{S_RING0 + 16}:{S_RING0 + 23}], s[{S_DP}:{S_DP + 1}], 0x40")
-else:
-    emit(f"s_load_dwordx16 s[{S_RING0 + 16}:{S_RING0 + 31}], s[{S_DP}:{S_DP + 1}], 0x40")
-emit(f"s_add_u32 s{S_DP}, s{S_DP}, {96 if LB == 2 else 128}")
+emit(f"s_load_dwordx16 s[{S_RING0 + 16}:{S_RING0 + 31}], s[{S_DP}:{S_DP + 1}], 0x40")
+emit(f"s_add_u32 s{S_DP}, s{S_DP}, 128")
 emit(f"s_addc_u32 s{S_DP + 1}, s{S_DP + 1}, 0")
 emit(f"s_mov_b32 s{S_CP}, %[chunk_lo]")
 emit(f"s_mov_b32 s{S_CP + 1}, %[chunk_hi]")
@@ -234,11 +188,8 @@ emit("s_waitcnt lgkmcnt(0)")
 for k in range(AHEAD):
     a_load(k)
 emit(f"s_waitcnt vmcnt({AHEAD})")                     # the copies of chunks 0, 1, 2 (issued before these loads) have landed
-if "barrier" not in ABL:
-    emit("s_barrier")
+emit("s_barrier")
 b_reads(0, 0)
-if LB == 2:
-    b_reads(1, 1)
 emit(f"s_getpc_b64 s[{S_BASE}:{S_BASE + 1}]")
 label("Lpc")
 emit(f"s_add_u32 s{S_BASE}, s{S_BASE}, Lb0_%=-Lpc_%=")
@@ -254,9 +205,9 @@ for J in range(8):
 label("Lend")                                         # offset END_OFF: the descriptor after the last op jumps here
 emit("s_waitcnt vmcnt(0) lgkmcnt(0)")
 
-clob = [f'"v{i}"' for i in range(V_B0, V_COPY + 1)] + [f'"s{i}"' for i in range(S_RING0, S_LAST + 2)] + ['"vcc"', '"scc"', '"memory"']
-print(f"// generated by gen_sweep_loop.py --ahead {AHEAD} --lds-ahead {LB}" + (f" --ablate {args.ablate}" if ABL else "") + "; do not edit")
-print(f"static_assert(SWEEP_LDS_AHEAD == {LB}, \"regenerate spmm_sweep_loop.inc\");")
+clob = ([f'"v{i}"' for i in range(V_B0, V_COPY + 1)] + [f'"s{i}"' for i in range(S_RING0, S_LAST + 2)] +
+        [f'"a{i}"' for i in range(128)] + ['"vcc"', '"scc"', '"memory"'])
+print("// generated by gen_sweep_loop.py; do not edit")
 print(f"static_assert(SWEEP_AHEAD == {AHEAD} && SWEEP_BLOCK_BYTES == {BLOCK_BYTES} && SWEEP_MARK_BASE == {MARK_BASE} && "
       f"SWEEP_MARK_BYTES == {MARK_BYTES} && SWEEP_END_OFF == {END_OFF}, \"regenerate spmm_sweep_loop.inc\");")
 print("asm volatile(")

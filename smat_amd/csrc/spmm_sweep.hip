@@ -116,10 +116,7 @@ __global__ __launch_bounds__(THREADS) void spmm_sweep_kernel(
     // A workgroup takes the tiles vb = blockIdx.x, blockIdx.x + gridDim.x, ... of the virtual grid n_vb.
     const int total = n_rg * n_panels;
     const int per_xcd = n_vb >> 3;
-#ifndef SWEEP_RGB
-#define SWEEP_RGB 4
-#endif
-    constexpr int RGB = SWEEP_RGB;
+    constexpr int RGB = 4;
     const int n_blk = (n_rg + RGB - 1) / RGB;
     bool zeros_written = false;
   for (int vb = blockIdx.x; vb < n_vb; vb += gridDim.x) {
@@ -217,10 +214,7 @@ __global__ __launch_bounds__(THREADS) void spmm_sweep_kernel(
         const uint32_t op_hi = __builtin_amdgcn_readfirstlane((uint32_t)((uintptr_t)op_base >> 32));
         const uint32_t chunk_lo = __builtin_amdgcn_readfirstlane((uint32_t)(uintptr_t)chunk_ptr);
         const uint32_t chunk_hi = __builtin_amdgcn_readfirstlane((uint32_t)((uintptr_t)chunk_ptr >> 32));
-#ifndef SWEEP_LOOP_INC
-#define SWEEP_LOOP_INC "spmm_sweep_loop.inc"
-#endif
-#include SWEEP_LOOP_INC
+#include "spmm_sweep_loop.inc"
     }
     asm volatile("s_nop 15\n\ts_nop 15" ::: "memory"); // the last MFMAs retire before their results are read
 
@@ -273,9 +267,6 @@ hipError_t launch_sweep(const SweepArgs &a, hipStream_t st)
     // workgroup keeps its CU and takes its tiles one after the other, which saves the dispatch of the later
     // ones and lets the stores of a tile drain while the next one fetches its first chunks.
     long launched = wgs;
-#ifdef SWEEP_PERSISTENT_GRID
-    if (SWEEP_PERSISTENT_GRID > 0 && launched > SWEEP_PERSISTENT_GRID) launched = SWEEP_PERSISTENT_GRID;
-#else
     {
         int dev = 0, cus = 0;
         if (hipGetDevice(&dev) == hipSuccess &&
@@ -284,7 +275,6 @@ hipError_t launch_sweep(const SweepArgs &a, hipStream_t st)
             if (launched > resident) launched = resident;
         }
     }
-#endif
     dim3 grid((unsigned)launched), block(THREADS);
     if (a.c_f32)
         hipLaunchKernelGGL((spmm_sweep_kernel<true>), grid, block, lds_bytes, st, a.vals, a.B, a.C,

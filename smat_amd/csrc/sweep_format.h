@@ -12,14 +12,8 @@ constexpr int SWEEP_WAVES = 8;   // wavefronts per workgroup
 constexpr int SWEEP_G = SWEEP_RW * SWEEP_WAVES; // 64 block rows per workgroup
 constexpr int SWEEP_S = 16;      // block columns (slabs) per K chunk
 constexpr int SWEEP_STAGES = 4;  // chunks resident in LDS
-#ifndef SWEEP_AHEAD_VALUE
-#define SWEEP_AHEAD_VALUE 4
-#endif
-constexpr int SWEEP_AHEAD = SWEEP_AHEAD_VALUE; // an A operand is loaded this many stream positions before its op
-#ifndef SWEEP_LDS_AHEAD_VALUE
-#define SWEEP_LDS_AHEAD_VALUE 1
-#endif
-constexpr int SWEEP_LDS_AHEAD = SWEEP_LDS_AHEAD_VALUE; // the B operands of an op are read from LDS this many stream positions before it
+constexpr int SWEEP_AHEAD = 4; // an A operand is loaded this many stream positions before its op
+constexpr int SWEEP_LDS_AHEAD = 1; // the B operands of an op are read from LDS this many stream positions before it
 constexpr int SWEEP_COPIES = 4;  // copy instructions per wavefront and chunk
 constexpr int SWEEP_MIN_OPS = SWEEP_AHEAD - 1 > SWEEP_COPIES ? SWEEP_AHEAD - 1 : SWEEP_COPIES; // ops per wavefront and chunk: two markers are at least AHEAD positions apart, and a marker finds the copies of the marker before it older than the A loads of the MIN_OPS + 1 positions since
 constexpr int SWEEP_OP_PAD = 16;   // descriptors after the end of the last stream (loaded ahead, never executed)
@@ -45,10 +39,7 @@ struct SweepOp {
 };
 constexpr uint32_t SWEEP_STAGE_BYTES = 32768;
 constexpr uint32_t SWEEP_ZERO_OFF = SWEEP_STAGES * SWEEP_STAGE_BYTES; // 131072
-#ifndef SWEEP_BLOCK_BYTES_VALUE
-#define SWEEP_BLOCK_BYTES_VALUE 128
-#endif
-constexpr uint32_t SWEEP_BLOCK_BYTES = SWEEP_BLOCK_BYTES_VALUE;
+constexpr uint32_t SWEEP_BLOCK_BYTES = 128;
 constexpr uint32_t SWEEP_MARK_BASE = 8 * 8 * 2 * SWEEP_BLOCK_BYTES;   // 16384
 constexpr uint32_t SWEEP_MARK_BYTES = 512;
 constexpr uint32_t SWEEP_END_OFF = SWEEP_MARK_BASE + 8 * SWEEP_MARK_BYTES;

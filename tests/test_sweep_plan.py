@@ -225,3 +225,19 @@ def test_headline_matrix_pairs_nearly_everything():
     assert plan["period_max_sum"] * WAVES < 1.08 * (plan["pairs"] + plan["singles"] + plan["fillers"])
     per_wave = np.diff(plan["op_ptr"])
     assert per_wave.min() >= 4 * 32 + 32 and per_wave.max() <= 72 * 32
+
+
+def test_committed_interpreter_loop_is_what_the_generator_writes():
+    """spmm_sweep_loop.inc is generated code kept in the repository: it has to be the output of the generator
+    next to it, and the generator takes no switches (the build makes the same comparison)."""
+    import os
+    import subprocess
+    import sys
+    csrc = os.path.join(os.path.dirname(os.path.dirname(os.path.abspath(__file__))), "smat_amd", "csrc")
+    run = subprocess.run([sys.executable, os.path.join(csrc, "gen_sweep_loop.py")], capture_output=True, text=True, check=True)
+    with open(os.path.join(csrc, "spmm_sweep_loop.inc")) as f:
+        committed = f.read()
+    assert run.stdout == committed
+    assert committed.splitlines()[0] == "// generated by gen_sweep_loop.py; do not edit"
+    bad = subprocess.run([sys.executable, os.path.join(csrc, "gen_sweep_loop.py"), "--ablate", "mfma"], capture_output=True, text=True)
+    assert bad.returncode != 0 and bad.stdout == ""
