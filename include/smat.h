@@ -115,12 +115,16 @@ typedef struct smat_plan smat_plan;
 /* row_ptr_host: the HOST copy of the BCSR row pointer (M/16+1 entries).
  * col_idx_host: HOST copy of the BCSR column index (may be NULL unless
  *               opts->kernel requests SMAT_KERNEL_SWEEP; without it SMAT_KERNEL_AUTO
- *               never chooses that kernel).
+ *               never chooses that kernel).  The sweep kernel needs the columns of every
+ *               block row strictly ascending, as csrToBcsr emits them (matrix.h:441-463):
+ *               otherwise SMAT_KERNEL_SWEEP / SMAT_KERNEL_MIXED are refused with
+ *               SMAT_ERR_INVALID and SMAT_KERNEL_AUTO stays with the row-wise kernel, which
+ *               takes the blocks of a row in any order (as mmaCBT.cu:44-66 does).
  * n_hint: the N the plan will mostly be used with (panel width choice). */
 int smat_plan_create(smat_plan **plan, const int32_t *row_ptr_host, const int32_t *col_idx_host,
                      size_t M, size_t K, size_t nnzb, size_t n_hint, const smat_spmm_opts *opts);
 /* Optional: lets the plan look at the block values (DEVICE arrays of the matrix the plan was
- * made for; row_ptr_host as in smat_plan_create).  The plan lists the nonzero columns of every
+ * made for; row_ptr_host must equal the array given to smat_plan_create, else SMAT_ERR_INVALID).  The plan lists the nonzero columns of every
  * block and keeps a COPY of them (32 bytes per nonzero column, in MFMA operand order), so that
  * SMAT_KERNEL_COMPACT multiplies only those and touches only the rows of B under them; with
  * SMAT_KERNEL_AUTO the plan switches to that kernel when fewer than 60% of the block columns

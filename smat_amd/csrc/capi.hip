@@ -54,6 +54,7 @@ struct smat_plan {
     };
     SweepDev sweep;       // all block rows (SMAT_KERNEL_SWEEP)
     SweepDev sweep_dense; // mixed dispatch: the block rows with mostly full blocks, when they fill the device
+    std::vector<int32_t> row_ptr_host; // the block row pointer the plan was made from: smat_plan_attach_values works from this copy
     std::vector<int32_t> col_idx_host; // kept for the split of a mixed plan (plans made with col_idx_host for AUTO / MIXED)
     uint64_t fingerprint = 0; // FNV-1a over row_ptr_host and, when given, col_idx_host
     bool fingerprint_has_cols = false;
@@ -373,11 +374,25 @@ static int smat_plan_create_impl(smat_plan **out, const int32_t *row_ptr_host,
     if (want == SMAT_KERNEL_SWEEP && !col_idx_host)
         return set_error(SMAT_ERR_INVALID, "SMAT_KERNEL_SWEEP needs col_idx_host");
     const size_t kb = K / 16;
-    if (col_idx_host)
+    // The sweep kernel pairs neighbouring blocks of a block row and schedules them by the K chunk they sit in:
+    // it needs the columns of a block row strictly ascending, as csrToBcsr emits them (matrix.h:441-463).  The
+    // row-wise kernel does not care about the order (like mmaCBT.cu:44-66).
+    bool cols_ascending = true;
+    if (col_idx_host) {
         for (size_t p = 0; p < nnzb; p++)
             if (col_idx_host[p] < 0 || col_idx_host[p] % 16 || (size_t)col_idx_host[p] >= K)
                 return set_error(SMAT_ERR_INVALID, "col_idx_host[%zu] = %d is not a block column of K = %zu",
                                  p, col_idx_host[p], K);
+        for (size_t i = 0; i < mb && cols_ascending; i++)
+            for (int32_t p = row_ptr_host[i] + 1; p < row_ptr_host[i + 1]; p++)
+                if (col_idx_host[p] <= col_idx_host[p - 1]) {
+                    cols_ascending = false;
+                    break;
+                }
+        if (!cols_ascending && (want == SMAT_KERNEL_SWEEP || want == SMAT_KERNEL_MIXED))
+            return set_error(SMAT_ERR_INVALID, "col_idx_host must be strictly ascending inside every block row for "
+                                               "SMAT_KERNEL_SWEEP / SMAT_KERNEL_MIXED");
+    }
 
     smat_plan *p = new (std::nothrow) smat_plan();
     if (!p) return set_error(SMAT_ERR_NOMEM, "out of host memory");
@@ -386,7 +401,8 @@ static int smat_plan_create_impl(smat_plan **out, const int32_t *row_ptr_host,
     p->kernel_requested = want;
     p->fingerprint = pattern_fingerprint(row_ptr_host, col_idx_host, mb, nnzb);
     p->fingerprint_has_cols = col_idx_host != nullptr;
-    if (col_idx_host && (want == SMAT_KERNEL_AUTO || want == SMAT_KERNEL_MIXED)) p->col_idx_host.assign(col_idx_host, col_idx_host + nnzb);
+    p->row_ptr_host.assign(row_ptr_host, row_ptr_host + mb + 1);
+    if (col_idx_host && cols_ascending && (want == SMAT_KERNEL_AUTO || want == SMAT_KERNEL_MIXED)) p->col_idx_host.assign(col_idx_host, col_idx_host + nnzb);
 
     // A block row is split when it is much longer than the average: chunks of
     // `chunk` blocks (even, so block pairs stay aligned with the MFMA K = 32).
@@ -436,7 +452,7 @@ static int smat_plan_create_impl(smat_plan **out, const int32_t *row_ptr_host,
     // rows x panels of 128 columns) fill the 256 CUs, and loses (0.3x .. 0.9x) when they do not.
     if (e == hipSuccess && opts && opts->b_layout == SMAT_B_ROW_MAJOR) e = dev_malloc(&p->d_bcol, K * n_hint * sizeof(uint16_t));
     bool sweep = want == SMAT_KERNEL_SWEEP;
-    if (want == SMAT_KERNEL_AUTO && col_idx_host && sweep_fills_device(mb, n_hint) &&
+    if (want == SMAT_KERNEL_AUTO && col_idx_host && cols_ascending && sweep_fills_device(mb, n_hint) &&
         (double)nnzb >= 0.05 * (double)mb * (double)kb)
         sweep = true;
     if (sweep && (nnzb >= (size_t)1 << 23 || nnzb < 2)) { // blocks are addressed in pairs, with 32-bit byte offsets
@@ -473,6 +489,11 @@ static int smat_plan_attach_values_impl(smat_plan *p, const uint16_t *vals, cons
 {
     if (!p || !row_ptr || !row_ptr_host) return set_error(SMAT_ERR_INVALID, "plan, row_ptr and row_ptr_host must not be NULL");
     if (p->nnzb && (!vals || !col_idx)) return set_error(SMAT_ERR_INVALID, "vals and col_idx must not be NULL");
+    // the work lists below index the plan's copy of col_idx_host through the row pointer: it has to be the one the
+    // plan was made from, not a stale or foreign array of the caller
+    if (memcmp(row_ptr_host, p->row_ptr_host.data(), p->row_ptr_host.size() * sizeof(int32_t)) != 0)
+        return set_error(SMAT_ERR_INVALID, "row_ptr_host differs from the block row pointer the plan was created with");
+    row_ptr_host = p->row_ptr_host.data();
     // The new list is built before the old one goes.  Whatever happens below, the old list describes values
     // that have changed, so it is dropped, and a plan left without a list goes back to a dense kernel.
     const size_t mb = p->M / 16;

@@ -58,3 +58,21 @@ def test_plan_argument_checks(smat):
         smat.Plan(rp, 32, 32, 3, 12)
     with pytest.raises(smat.SmatError):  # col_idx not a block column
         smat.Plan(rp, 32, 32, 3, 64, col_idx_host=np.array([0, 8, 16], np.int32))
+
+
+def test_sweep_plan_refuses_columns_that_do_not_ascend(smat):
+    """The sweep kernel pairs neighbouring blocks of a block row by the K chunk they sit in: columns that are not
+    strictly ascending inside a block row are refused when such a plan is asked for (before any device work)."""
+    from smat_amd import generators as gen
+    A = gen.random_bcsr(64, 160, 0.1, seed=3)
+    rp, ci = A["b_row_ptr"], A["b_col_idx"].copy()
+    for i in range(64):  # the columns of every block row in descending order
+        ci[rp[i]:rp[i + 1]] = ci[rp[i]:rp[i + 1]][::-1]
+    for kernel in (smat.KERNEL_SWEEP, smat.KERNEL_MIXED):
+        with pytest.raises(smat.SmatError) as err:
+            smat.Plan(rp, A["M"], A["K"], A["nnzb"], 4096, col_idx_host=ci, kernel=kernel)
+        assert err.value.code == -1 and "ascending" in str(err.value)
+    dup = A["b_col_idx"].copy()
+    dup[rp[5] + 1] = dup[rp[5]]  # a repeated column is no better
+    with pytest.raises(smat.SmatError):
+        smat.Plan(rp, A["M"], A["K"], A["nnzb"], 4096, col_idx_host=dup, kernel=smat.KERNEL_SWEEP)

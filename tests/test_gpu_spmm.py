@@ -247,6 +247,29 @@ def test_sweep_kernel_skewed_and_empty_rows(smat, cuda, oracle):
     assert not C.reshape(A["M"], N)[0:16].any()
 
 
+def test_unsorted_block_columns_take_the_row_wise_kernel(smat, cuda, oracle):
+    """Block columns in descending order inside the block rows: the kernel choice left to the plan falls back to the
+    row-wise kernel (which, like the reference, does not care about the order) instead of the sweep kernel."""
+    A = gen.random_bcsr(512, 64, 0.2, seed=77)
+    rp = A["b_row_ptr"]
+    ci, val = A["b_col_idx"].copy(), A["b_val"].reshape(-1, 256).copy()
+    for i in range(A["M"] // 16):
+        ci[rp[i]:rp[i + 1]] = ci[rp[i]:rp[i + 1]][::-1]
+        val[rp[i]:rp[i + 1]] = val[rp[i]:rp[i + 1]][::-1]
+    N = 2048  # 8 row groups x 32 panels: the sweep kernel would be the plan's choice for ascending columns
+    B = gen.dense_b(A["K"], N, seed=5)
+    ref = oracle_ref(oracle, A, B, N)
+    p = smat.Plan(rp, A["M"], A["K"], A["nnzb"], N, col_idx_host=A["b_col_idx"])
+    assert p.info()["kernel"] == SWEEP
+    p.close()
+    p = smat.Plan(rp, A["M"], A["K"], A["nnzb"], N, col_idx_host=ci)
+    assert p.info()["kernel"] == 1
+    p.close()
+    Ar = dict(A, b_col_idx=ci, b_val=val.reshape(-1))
+    C = gpu_spmm(smat, cuda, Ar, B, N, plan=True)
+    assert oracle.compare(C, ref)[0] <= TOL_F16
+
+
 def test_sweep_needs_a_plan_with_col_idx(smat, cuda):
     A = gen.random_bcsr(4, 4, 0.5, seed=1)
     with pytest.raises(smat.SmatError):
