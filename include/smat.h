@@ -158,11 +158,12 @@ int smat_plan_info(const smat_plan *plan, int64_t *info);
  * rows, one wavefront each).
  * Non-finite inputs: one MFMA covers two blocks.  The row-wise kernel multiplies an unpaired
  * block together with a block of zeros, the compact kernel pads a block row with zero columns
- * (0 x Inf = NaN where B holds Inf or NaN).  The sweep kernel multiplies an unpaired block together
- * with the block that follows it in vals (the one before it for the last block) and 16 rows of zeros
- * in place of B, and its filler ops multiply blocks 0 and 1 by zeros: where vals holds Inf or NaN, a
- * row of C that another block row's block shares an MFMA with can come out NaN.  A block-by-block
- * product (mmaCBT.cu:44-66) gives Inf / NaN only where the operands of that element hold them.
+ * (0 x Inf = NaN where B holds Inf or NaN).  The sweep kernel multiplies an unpaired block together with
+ * a neighbouring block of the SAME block row and 16 rows of zeros in place of B, and its filler ops multiply two
+ * blocks of the block row they add to by zeros: an Inf or NaN in vals stays in its own block row of C (where a
+ * block-by-block product, mmaCBT.cu:44-66, has an Inf or NaN as well).  Only a block that is alone in its block
+ * row shares its MFMA with the block that follows it in vals (another row's), and a wavefront whose block rows all
+ * have fewer than two blocks uses blocks 0 and 1 for its fillers: Inf or NaN in THOSE blocks can turn that row NaN.
  * Finite inputs give the same sums up to the fp32 summation order. */
 int smat_spmm_bcsr_f16_ex(const uint16_t *vals, const int32_t *row_ptr, const int32_t *col_idx,
                           const uint16_t *B, void *C, size_t M, size_t N, size_t K, size_t nnzb,

@@ -76,11 +76,21 @@ void build_sweep_plan(const int32_t *row_ptr, const int32_t *col_idx, size_t mb,
                         pair = true;
                     }
                 }
-                if (!pair) { // the other half of the MFMA reads zeros instead of rows of B
-                    if (q + 1 < nnzb) { // blocks (q, q + 1) are loaded, the second multiplies zeros
+                if (!pair) {
+                    // The other half of the MFMA reads zeros instead of rows of B, but the load brings two
+                    // neighbouring blocks: take the neighbour from the SAME block row where the row has one, so that
+                    // an Inf or NaN in another row's values (times zero: NaN) cannot reach this row of C.
+                    if (q + 1 < q_end) { // blocks (q, q + 1), the second multiplies zeros
                         op.w0 = (uint32_t)q * 512u;
                         op.w2 = SWEEP_ZERO_OFF - off0;
-                    } else { // last block of the matrix: blocks (q - 1, q), the first multiplies zeros
+                    } else if (q > row_ptr[br]) { // last block of its row: blocks (q - 1, q), the first multiplies zeros
+                        op.w0 = (uint32_t)(q - 1) * 512u;
+                        op.w1 = SWEEP_ZERO_OFF;
+                        op.w2 = off0 - SWEEP_ZERO_OFF;
+                    } else if (q + 1 < nnzb) { // the only block of its row: the neighbour is another row's
+                        op.w0 = (uint32_t)q * 512u;
+                        op.w2 = SWEEP_ZERO_OFF - off0;
+                    } else { // and the last block of the matrix: the read stays inside vals
                         op.w0 = (uint32_t)(q - 1) * 512u;
                         op.w1 = SWEEP_ZERO_OFF;
                         op.w2 = off0 - SWEEP_ZERO_OFF;
@@ -220,7 +230,19 @@ void build_sweep_plan(const int32_t *row_ptr, const int32_t *col_idx, size_t mb,
             by_chunk = schedule[(size_t)w];
             struct Item { int kind, row; SweepOpHost op; }; // kind: 0 op, 1 marker, 2 end
             std::vector<Item> items;
-            const SweepOpHost idle{0, SWEEP_ZERO_OFF, 0, 0}; // blocks 0 and 1 times zeros
+            const SweepOpHost idle{0, SWEEP_ZERO_OFF, 0, 0}; // markers and the end: no blocks of their own
+            // A filler op multiplies two blocks by zeros and adds the result to one of the wavefront's block rows:
+            // two blocks of that very row (then an Inf or NaN in them is in that row of C anyway), blocks 0 and 1
+            // of the matrix only when no row of the wavefront has two.
+            Item filler{0, 0, idle};
+            for (int r = 0; r < RW; r++) {
+                const int32_t br = out.row_map[(rg * WAVES + (size_t)w) * RW + (size_t)r];
+                if (br >= 0 && row_ptr[br + 1] - row_ptr[br] >= 2) {
+                    filler.row = r;
+                    filler.op.w0 = (uint32_t)row_ptr[br] * 512u;
+                    break;
+                }
+            }
             for (size_t c = 0; c < n_chunks; c++) {
                 std::vector<Ranked> &list = by_chunk[c];
                 std::stable_sort(list.begin(), list.end(), [](const Ranked &a, const Ranked &b) {
@@ -234,7 +256,7 @@ void build_sweep_plan(const int32_t *row_ptr, const int32_t *col_idx, size_t mb,
                     size_t ok = 0;
                     while (ok < list.size() && list[ok].hi > (int32_t)c) ok++;
                     if (ok == list.size()) {
-                        items.push_back(Item{0, 0, idle});
+                        items.push_back(filler);
                         out.n_fillers++;
                     } else if (ok > 0) {
                         std::rotate(list.begin(), list.begin() + (long)ok, list.begin() + (long)ok + 1);
@@ -242,7 +264,7 @@ void build_sweep_plan(const int32_t *row_ptr, const int32_t *col_idx, size_t mb,
                 }
                 for (const Ranked &x : list) items.push_back(Item{0, x.row, x.op});
                 for (size_t k = list.size(); k < (size_t)MIN_OPS; k++) { // filler ops keep the markers AHEAD positions apart
-                    items.push_back(Item{0, 0, idle});
+                    items.push_back(filler);
                     out.n_fillers++;
                 }
             }
@@ -288,18 +310,18 @@ void build_sweep_plan(const int32_t *row_ptr, const int32_t *col_idx, size_t mb,
 
 } // namespace smat
 
-// Test hook (not part of smat.h): builds the work list on the host and hands it out.  Arrays are
+// Test hook (not part of smat.h): builds the work list on the host (rows != NULL: of these block rows only) and hands it out.  Arrays are
 // allocated with malloc; release each with smat_host_free.  row_map: n_rg * 64 block rows (-1 = none).  counts[0..5] = row groups, listed
 // chunks, stream entries (ops, fillers, markers, ends; without padding), pairs, singles, fillers.
 static int smat_internal_sweep_plan_impl(const int32_t *row_ptr, const int32_t *col_idx, size_t M, size_t K,
-                                         int32_t **rg_chunk_ptr, int32_t **chunk_ids, int32_t **op_ptr,
+                                         const int32_t *rows, size_t n_rows, int32_t **rg_chunk_ptr, int32_t **chunk_ids, int32_t **op_ptr,
                                          uint32_t **ops, int32_t **row_map, int64_t *counts)
 {
     if (!row_ptr || !col_idx || !rg_chunk_ptr || !chunk_ids || !op_ptr || !ops || !row_map || !counts) return SMAT_ERR_INVALID;
     if (M == 0 || M % 16 || K % 16 || row_ptr[M / 16] < 2) return SMAT_ERR_INVALID;
     smat::SweepPlanHost p;
     try {
-        smat::build_sweep_plan(row_ptr, col_idx, M / 16, K / 16, p);
+        smat::build_sweep_plan(row_ptr, col_idx, M / 16, K / 16, p, rows, n_rows);
     } catch (...) {
         return SMAT_ERR_NOMEM;
     }
@@ -330,8 +352,8 @@ extern "C" void smat_internal_sweep_params(int32_t *out)
 }
 
 extern "C" int smat_internal_sweep_plan(const int32_t *row_ptr, const int32_t *col_idx, size_t M, size_t K,
-                                         int32_t **rg_chunk_ptr, int32_t **chunk_ids, int32_t **op_ptr,
+                                         const int32_t *rows, size_t n_rows, int32_t **rg_chunk_ptr, int32_t **chunk_ids, int32_t **op_ptr,
                                          uint32_t **ops, int32_t **row_map, int64_t *counts)
 {
-    return smat::guarded("smat_internal_sweep_plan", [&] { return smat_internal_sweep_plan_impl(row_ptr, col_idx, M, K, rg_chunk_ptr, chunk_ids, op_ptr, ops, row_map, counts); });
+    return smat::guarded("smat_internal_sweep_plan", [&] { return smat_internal_sweep_plan_impl(row_ptr, col_idx, M, K, rows, n_rows, rg_chunk_ptr, chunk_ids, op_ptr, ops, row_map, counts); });
 }

@@ -270,6 +270,36 @@ def test_unsorted_block_columns_take_the_row_wise_kernel(smat, cuda, oracle):
     assert oracle.compare(C, ref)[0] <= TOL_F16
 
 
+def test_sweep_kernel_keeps_non_finite_values_inside_their_block_row(smat, cuda, oracle):
+    """An unpaired block shares its MFMA with a neighbouring block times zeros, a filler op multiplies two blocks by
+    zeros: the plan takes those blocks from the same block row, so Inf in the values of one block row (times zero:
+    NaN) does not reach any other row of C.  Every third block row is all Inf here; the others must come out as
+    the oracle computes them (every row has at least two blocks)."""
+    rng = np.random.default_rng(9)
+    lengths = rng.integers(2, 9, size=130).tolist()  # few blocks per row over 100 block columns: many unpaired blocks and fillers
+    A = gen.random_bcsr(130, 100, 0.0, seed=21, row_lengths=lengths)
+    N = 128
+    B = gen.dense_b(A["K"], N, seed=22, dist="normal")
+    ref = oracle_ref(oracle, A, B, N).reshape(A["M"], N)
+    val = A["b_val"].reshape(-1, 256).copy()
+    rp = A["b_row_ptr"]
+    bad_rows = np.arange(1, 130, 3)
+    for r in bad_rows:
+        val[rp[r]:rp[r + 1]] = 0x7C00  # +Inf
+    Ainf = dict(A, b_val=val.reshape(-1))
+    p = smat.Plan(rp, A["M"], A["K"], A["nnzb"], N, col_idx_host=A["b_col_idx"], kernel=SWEEP)
+    info = p.info()
+    p.close()
+    assert info["sweep_ops"] > 0
+    C = gpu_spmm(smat, cuda, Ainf, B, N, plan=True, kernel=SWEEP).reshape(A["M"], N)
+    good = np.ones(A["M"], bool)
+    for r in bad_rows:
+        good[r * 16:r * 16 + 16] = False
+    assert np.isfinite(C[good].view(np.float16)).all()
+    assert oracle.compare(np.ascontiguousarray(C[good]), np.ascontiguousarray(ref[good]))[0] <= TOL_F16
+    assert not np.isfinite(C[~good].view(np.float16)).any()  # Inf x B: Inf or NaN, as a block-by-block product gives
+
+
 def test_sweep_needs_a_plan_with_col_idx(smat, cuda):
     A = gen.random_bcsr(4, 4, 0.5, seed=1)
     with pytest.raises(smat.SmatError):

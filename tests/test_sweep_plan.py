@@ -25,15 +25,18 @@ LDS_MASK = 0x1C0E0
 PAD, CHUNK_PAD = 16, 4
 
 
-def sweep_plan(row_ptr, col_idx, M, K):
+def sweep_plan(row_ptr, col_idx, M, K, rows=None):
+    """rows: the ascending block rows the plan is made for (what mixed dispatch hands to the sweep kernel); None = all."""
     fn = lib.smat_internal_sweep_plan
     fn.restype = C.c_int
-    fn.argtypes = [C.c_void_p, C.c_void_p, C.c_size_t, C.c_size_t] + [C.POINTER(C.c_void_p)] * 5 + [C.POINTER(C.c_int64)]
+    fn.argtypes = [C.c_void_p, C.c_void_p, C.c_size_t, C.c_size_t, C.c_void_p, C.c_size_t] + [C.POINTER(C.c_void_p)] * 5 + [C.POINTER(C.c_int64)]
     row_ptr = np.ascontiguousarray(row_ptr, np.int32)
     col_idx = np.ascontiguousarray(col_idx, np.int32)
+    rows_arr = None if rows is None else np.ascontiguousarray(rows, np.int32)
     out = [C.c_void_p() for _ in range(5)]
     counts = (C.c_int64 * 6)()
-    rc = fn(row_ptr.ctypes.data, col_idx.ctypes.data, M, K, *[C.byref(o) for o in out], counts)
+    rc = fn(row_ptr.ctypes.data, col_idx.ctypes.data, M, K, None if rows is None else rows_arr.ctypes.data,
+            0 if rows is None else rows_arr.size, *[C.byref(o) for o in out], counts)
     assert rc == 0
     n_rg, n_chunks, n_ops = counts[0], counts[1], counts[2]
 
@@ -70,8 +73,9 @@ def slot_of(off):
     return slot // S, slot % S
 
 
-def replay(plan, A, Bd):
-    """Runs the streams on dense numpy operands. A: dict from gen (BCSR), Bd: K x N float64."""
+def replay(plan, A, Bd, rows=None):
+    """Runs the streams on dense numpy operands. A: dict from gen (BCSR), Bd: K x N float64.  rows: the block rows
+    the plan was made for (None = all): only their blocks may be used, 64 of them to a row group in this order."""
     M, K, rp, ci = A["M"], A["K"], A["b_row_ptr"], A["b_col_idx"]
     blocks = A["b_val"].view(np.float16).astype(np.float64).reshape(-1, 16, 16)
     nnzb = ci.size
@@ -80,6 +84,9 @@ def replay(plan, A, Bd):
     block_row = np.repeat(np.arange(M // 16), np.diff(rp))
     n_rg = plan["rg_chunk_ptr"].size - 1
     n_real = n_fill = 0
+    subset = np.arange(M // 16) if rows is None else np.asarray(rows)
+    place = {int(br): i for i, br in enumerate(subset)}  # block row -> position in the plan's list of rows
+    row_len = np.diff(rp)
     for rg in range(n_rg):
         chunks = plan["chunk_ids"][plan["rg_chunk_ptr"][rg]:plan["rg_chunk_ptr"][rg + 1]]
         assert np.all(np.diff(chunks) > 0)
@@ -133,9 +140,20 @@ def replay(plan, A, Bd):
                 off_lo, off_hi = w1, (w1 + int(np.int32(np.uint32(w2)))) & 0xFFFFFFFF
                 if off_lo == ZERO_OFF and off_hi == ZERO_OFF:
                     n_fill += 1
+                    # a filler adds two blocks times zeros to block row br: they are that row's own blocks, unless
+                    # no row of this wavefront has two (then blocks 0 and 1, which the kernel can always load)
+                    mine = plan["row_map"][(rg * WAVES + w) * RW:(rg * WAVES + w + 1) * RW]
+                    if any(b >= 0 and row_len[b] >= 2 for b in mine):
+                        assert br >= 0 and block_row[q] == br and block_row[q + 1] == br
+                    else:
+                        assert q == 0
                     continue
                 n_real += 1
-                assert 0 <= br < M // 16 and br // G == rg
+                assert br in place and place[br] // G == rg
+                # both loaded blocks belong to the op's block row, also when one of them multiplies zeros: only a
+                # block that is alone in its row travels with another row's block
+                if row_len[br] >= 2:
+                    assert block_row[q] == br and block_row[q + 1] == br
                 for half, off in enumerate((off_lo, off_hi)):
                     if off == ZERO_OFF:
                         continue
@@ -151,10 +169,14 @@ def replay(plan, A, Bd):
                     used[blk] += 1
                     Cd[br * 16:br * 16 + 16] += blocks[blk] @ Bd[k0:k0 + 16]
             assert ended and cur == chunks.size - 1 and in_chunk >= MIN_OPS
-    assert np.all(used == 1), "a block is multiplied zero or several times"
+    in_subset = np.isin(block_row, subset)
+    assert np.all(used[in_subset] == 1) and not used[~in_subset].any(), "a block is multiplied zero or several times, or is not the plan's"
     assert n_fill == plan["fillers"] and n_real == plan["pairs"] + plan["singles"]
-    rows = plan["row_map"][plan["row_map"] >= 0]
-    assert np.array_equal(np.sort(rows), np.arange(M // 16)), "row_map is not a partition of the block rows"
+    mapped = plan["row_map"][plan["row_map"] >= 0]
+    assert np.array_equal(np.sort(mapped), np.sort(subset)), "row_map is not a partition of the plan's block rows"
+    for rg in range(n_rg):  # row group rg holds the rows subset[64 rg : 64 rg + 64], the slots that are left say -1
+        got = plan["row_map"][rg * G:(rg + 1) * G]
+        assert np.array_equal(np.sort(got[got >= 0]), np.sort(subset[rg * G:(rg + 1) * G]))
     # read-ahead: the entries after the last stream exist and are harmless
     tail = plan["ops"][plan["n_entries"]:]
     assert tail.shape[0] == PAD and np.all(tail == np.array([0, ZERO_OFF, 0, END_OFF], np.uint32))
@@ -196,6 +218,36 @@ def test_replay_gives_a_times_b(mb, kb, density, seed):
     Cd = replay(plan, A, Bd)
     assert np.allclose(Cd, dense_of(A) @ Bd, rtol=1e-12, atol=1e-12)
     assert plan["pairs"] * 2 + plan["singles"] == A["nnzb"]
+
+
+@pytest.mark.parametrize("mb,kb,density,seed,pick", [(200, 64, 0.10, 11, "odd"), (150, 40, 0.3, 12, "random"), (300, 33, 0.05, 13, "blocks_of_3"),
+                                                      (70, 48, 0.2, 14, "one")])
+def test_replay_of_a_row_subset(mb, kb, density, seed, pick):
+    """The plan of mixed dispatch: only some block rows (interleaved with rows that another kernel takes), packed 64
+    to a row group.  Exactly their blocks are used, once each; an unpaired block never travels with a block of a
+    row outside the subset unless it is alone in its row; the last row group is partly empty."""
+    A = random_mask_matrix(mb, kb, density, seed, empty_rows=(1, 5), long_rows=(7,))
+    rng = np.random.default_rng(seed)
+    if pick == "odd":
+        rows = np.arange(1, mb, 2)
+    elif pick == "random":
+        rows = np.sort(rng.choice(mb, size=mb // 3, replace=False))
+    elif pick == "blocks_of_3":
+        rows = np.array([r for r in range(mb) if (r // 3) % 2 == 0])
+    else:
+        rows = np.array([7])
+    assert rows.size % G != 0  # the last row group has unused slots
+    plan = sweep_plan(A["b_row_ptr"], A["b_col_idx"], A["M"], A["K"], rows=rows)
+    Bd = rng.normal(size=(A["K"], 8))
+    Cd = replay(plan, A, Bd, rows=rows)
+    D = dense_of(A)
+    keep = np.zeros(A["M"], bool)
+    for r in rows:
+        keep[r * 16:r * 16 + 16] = True
+    D[~keep] = 0
+    assert np.allclose(Cd, D @ Bd, rtol=1e-12, atol=1e-12)
+    row_blocks = np.diff(A["b_row_ptr"])[rows].sum()
+    assert plan["pairs"] * 2 + plan["singles"] == row_blocks
 
 
 def test_single_last_block_is_listed_as_second_half():
