@@ -39,6 +39,7 @@
 #include <cstdlib>
 #include <cstring>
 #include <atomic>
+#include <chrono>
 #include <functional>
 #include <numeric>
 #include <thread>
@@ -441,8 +442,11 @@ private:
         for (;;) {
             int idle = 0;
             while (generation_.load(std::memory_order_acquire) == seen) {
+                // short gaps between jobs are spun through; in the long serial phases of a run the helpers
+                // give the core away and finally sleep, 50 us at a time
                 if (++idle < 4096) spin_pause();
-                else std::this_thread::yield();
+                else if (idle < 65536) std::this_thread::yield();
+                else std::this_thread::sleep_for(std::chrono::microseconds(50));
             }
             seen = generation_.load(std::memory_order_acquire);
             if (stop_.load(std::memory_order_acquire)) return;
@@ -686,6 +690,9 @@ std::vector<int64_t> keeper_grouping(int64_t rows, const int64_t *row_ptr, const
             ahead = Span{free_buffer(), behind, behind < rows ? batch_rows(behind, since_change + looked.count) : 0};
             set_job(stored, ahead);
             pool.start(job);
+            // whatever ends this iteration (an insertion that runs out of memory throws), the helpers have left the
+            // job before the buffers and the job itself go away
+            struct WaitOnExit { ScanPool &p; ~WaitOnExit() { p.wait(); } } wait_on_exit{pool};
             const float *res = results[looked.buf].data();
             int64_t x = 0;
             bool merged = false;
