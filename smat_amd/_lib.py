@@ -35,6 +35,7 @@ SIGNATURES = {
     "smat_last_error": (C.c_char_p, []),
     "smat_version": (C.c_char_p, []),
     "smat_spmm_bcsr_f16": (_int, [_vp, _vp, _vp, _vp, _vp, _sz, _sz, _sz, _sz, _vp, _vp]),
+    "smat_plan_cache_clear": (_int, []),
     "smat_spmm_bcsr_f16_ex": (_int, [_vp, _vp, _vp, _vp, _vp, _sz, _sz, _sz, _sz, C.POINTER(SpmmOpts), _vp]),
     "smat_spmm_bcsr_f16_static": (_int, [_vp, _vp, _vp, _vp, _vp, _sz, _sz, _sz, _sz, _vp]),
     "smat_plan_values_current": (_int, [_vp, _vp, C.POINTER(C.c_int)]),

@@ -250,15 +250,7 @@ extern "C" int smat_spmm_bcsr_f16_ex(const uint16_t *vals, const int32_t *row_pt
     return SMAT_OK;
 }
 
-extern "C" int smat_spmm_bcsr_f16(const uint16_t *vals, const int32_t *row_ptr,
-                                   const int32_t *col_idx, const uint16_t *B, uint16_t *C, size_t M,
-                                   size_t N, size_t K, size_t nnzb, const int32_t *block_info,
-                                   const int32_t *rel_map)
-{
-    (void)block_info;
-    (void)rel_map;
-    return smat_spmm_bcsr_f16_ex(vals, row_ptr, col_idx, B, C, M, N, K, nnzb, nullptr, nullptr);
-}
+// The drop-in entry point smat_spmm_bcsr_f16 lives in plan_cache.hip.
 
 // ---- SpMM without any allocation ------------------------------------------------
 // For callers that cannot allocate (HIP graph capture, serving loops, harnesses that forbid hipMalloc): the

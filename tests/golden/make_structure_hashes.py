@@ -6,7 +6,9 @@ column permutations of every benchmark workload, computed by this build on the m
 The tests and bench.py recompute the same hashes wherever they run (the GPU machine's host code and its
 device-side blocking) and compare: the structure must be the same bit for bit on every machine.  The reordered
 R-MAT scale 20 workload needs the permutations of an earlier smat_amd.reorder_csr run (ten minutes on eight
-threads); without --perm-file its entry is carried over from the existing file."""
+threads): they are read from rmat_s20_deg16_perms.npz next to this file unless --perm-file names another file.
+The "reference" records inside the entries (what the reference's own program made of the same patterns) are
+written by make_reference_structures.py and carried over here."""
 import argparse
 import json
 import os
@@ -20,7 +22,8 @@ import bench  # noqa: E402
 
 WORKLOADS = ["band_4096_bw64_N128", "er_16384_0.1pct_N256", "er_16384_0.1pct_reordered_N256", "rmat_s20_deg16_N128",
              "rmat_s20_deg16_reordered_N128", "block_pruned_8192_10pct_N4096", "half_pruned_half_er_8192_N4096",
-             "stencil27_64_N64", "stencil27_64_reordered_N64"]
+             "stencil27_64_N64", "stencil27_64_reordered_N64", "rmat_s15_deg16_reordered_N128", "rmat_s16_deg16_reordered_N128",
+             "rmat_s17_deg16_reordered_N128"]
 OUT = os.path.join(HERE, "structure_hashes.json")
 
 
@@ -35,6 +38,13 @@ def entry(name):
     return e
 
 
+def keep_reference(new, old):
+    """The "reference" record of an entry is written by make_reference_structures.py: carried over."""
+    if old and "reference" in old:
+        new["reference"] = old["reference"]
+    return new
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--perm-file", default=None)
@@ -43,11 +53,7 @@ def main():
     old = json.load(open(OUT)) if os.path.exists(OUT) else {}
     out = {}
     for name in WORKLOADS:
-        if name == "rmat_s20_deg16_reordered_N128" and not args.perm_file:
-            if name in old:
-                out[name] = old[name]
-            continue
-        out[name] = entry(name)
+        out[name] = keep_reference(entry(name), old.get(name))
         print(name, out[name], flush=True)
     with open(OUT, "w") as f:
         json.dump(out, f, indent=1, sort_keys=True)

@@ -80,6 +80,64 @@ def test_config3_rmat_scale20_full_size(smat, cuda, oracle):
     dev.close()
 
 
+@pytest.mark.timeout(900)
+def test_config3_rmat_scale20_reordered_full_size(smat, cuda, oracle):
+    """Config 3 in the form the benchmark states it: R-MAT scale 20 after both reorder passes (the permutations of
+    a ten-minute smat_reorder_csr run, tests/golden/rmat_s20_deg16_perms.npz), then 16 x 16 BCSR: 8,076,241 blocks
+    instead of 11,159,910.  The blocked structure has the recorded hash; sampled block rows (the heaviest and the
+    last ones among them) against the oracle; A (2 B) = 2 (A B) over the whole result; and the result is the
+    row-permuted product of the UNREORDERED matrix with the rows of B permuted back (on sampled rows)."""
+    import json
+    import os
+    import torch
+    import bench
+    name = "rmat_s20_deg16_reordered_N128"
+    bench.INFO.clear()
+    A, B, N = bench.build_workload(name)
+    want = json.load(open(bench.GOLDEN_STRUCTURE))[name]
+    M, K, nnzb = A["M"], A["K"], A["nnzb"]
+    assert (M, K, N, nnzb) == (want["M"], want["K"], want["N"], want["nnzb"]) and nnzb == 8076241
+    assert bench.sha256_of(A["b_row_ptr"].astype(np.int32), A["b_col_idx"].astype(np.int32)) == want["pattern_sha256"]
+    assert bench.INFO["perm_sha256"] == want["perm_sha256"]
+    mb = M // 16
+    heaviest = int(np.argmax(np.diff(A["b_row_ptr"])))
+    rows = sample_rows(mb, 12, extra=(heaviest, mb - 1, mb - 2))
+    B2 = (B.view(np.float16) * np.float16(2)).view(np.uint16)
+    vals, Bd, B2d = to_dev(torch, A["b_val"], cuda), to_dev(torch, B, cuda), to_dev(torch, B2, cuda)
+    rp, ci = to_dev(torch, A["b_row_ptr"].astype(np.int32), cuda), to_dev(torch, A["b_col_idx"].astype(np.int32), cuda)
+    plan = smat.Plan(A["b_row_ptr"], M, K, nnzb, N, col_idx_host=A["b_col_idx"], kernel=0)
+    plan.attach_values(vals, rp, ci)
+    assert plan.info()["kernel"] == 5
+    C = torch.full((M, N), 0x7E00, dtype=torch.int16, device=cuda)
+    smat.spmm(vals, rp, ci, Bd, C, M, N, K, nnzb, plan=plan)
+    C2 = torch.full((M, N), 0x7E00, dtype=torch.int16, device=cuda)
+    smat.spmm(vals, rp, ci, B2d, C2, M, N, K, nnzb, plan=plan)
+    torch.cuda.synchronize()
+    plan.close()
+    C_host = C.cpu().numpy().view(np.uint16)
+    check_sampled(oracle, A, B, N, C_host, rows)
+    c, c2 = C.view(torch.float16), C2.view(torch.float16)
+    assert bool(torch.isfinite(c2).all()) and float(c.abs().max()) < 30000
+    tiny = c.abs() < 2.0**-13
+    assert bool(((c * 2 == c2) | tiny).all())
+    del c, c2, C, C2, vals
+    # against the matrix before the reorder: row i of the result is row perm_rows[i] of (A_original x B_back), where
+    # B_back has the rows of B moved back to their old places.  Checked on the rows of the sampled block rows.
+    z = np.load(bench.RMAT20_PERMS)
+    pr, pc = z["perm_rows"].astype(np.int64), z["perm_cols"].astype(np.int64)
+    d = gen.rmat(20, 16)
+    Bm = B.reshape(N, K)
+    B_back = np.empty_like(Bm)
+    B_back[:, pc] = Bm
+    new_rows = np.concatenate([np.arange(16 * r, 16 * r + 16) for r in rows])
+    old_rows = pr[new_rows]
+    lens = (d["row_ptr"][old_rows + 1] - d["row_ptr"][old_rows]).astype(np.int64)
+    sel = np.concatenate([np.arange(d["row_ptr"][o], d["row_ptr"][o + 1]) for o in old_rows]) if lens.sum() else np.zeros(0, np.int64)
+    sub_rp = np.concatenate([[0], np.cumsum(lens)]).astype(np.int32)
+    ref = oracle.spmm_csr(new_rows.size, N, K, sub_rp, d["col_idx"][sel], d["val"][sel], B_back.ravel())
+    assert oracle.compare(np.ascontiguousarray(C_host[new_rows]), ref)[0] <= TOL_F16
+
+
 def test_config2_reordered_full_size(smat, cuda, oracle):
     """Config 2 (16384 x 16384, 0.1 %, N = 256) after both reorder passes: whole result against the oracle,
     and equal to the product of the unpermuted matrix with rows and B permuted accordingly."""

@@ -37,6 +37,8 @@ def gpu_spmm(smat, cuda, A, B_bits, N, plan=False, c_f32=False, drop_in=False, p
     if plan:
         p = smat.Plan(A["b_row_ptr"], M, K, nnzb, N, col_idx_host=A["b_col_idx"], kernel=kernel)
     torch.cuda.synchronize()
+    if drop_in:  # fresh tensors may sit where another test's matrix of the same size sat: no plan from before
+        smat.lib.smat_plan_cache_clear()
     smat.spmm(vals, rp, ci, B, C, M, N, K, nnzb, plan=p, c_f32=c_f32, drop_in=drop_in, kernel=kernel)
     torch.cuda.synchronize()
     out = C.cpu().numpy()
@@ -139,6 +141,96 @@ def test_drop_in_entry_matches_options_entry(smat, cuda, oracle):
     c2 = gpu_spmm(smat, cuda, A, B, N, drop_in=False)
     assert np.array_equal(c1, c2)
     assert oracle.compare(c1, oracle_ref(oracle, A, B, N))[0] <= TOL_F16
+
+
+def cache_stats(smat):
+    import ctypes as C
+    out = (C.c_int64 * 4)()
+    smat.lib.smat_internal_plan_cache_stats(out)
+    return {"built": out[0], "hits": out[1], "rebuilt": out[2], "entries": out[3]}
+
+
+def test_drop_in_entry_point_keeps_a_plan_per_matrix(smat, cuda, oracle, monkeypatch):
+    """smat_spmm_bcsr_f16 (the reference's positional signature, no plan argument) makes a plan on its first call
+    with a matrix and reuses it: two matrices in turn, each result bit for bit what an explicit plan gives; a
+    pattern rewritten in place is caught by the checksum (or by smat_plan_cache_clear); SMAT_PLAN_CACHE=0 goes back
+    to plain launches."""
+    import ctypes as C
+    import torch
+    lib = smat.lib
+    lib.smat_plan_cache_clear()
+    lib.smat_internal_plan_cache_check_every(C.c_uint64(0))
+
+    def setup(A, N, seed):
+        B = gen.dense_b(A["K"], N, seed=seed, dist="normal")
+        t = {"A": A, "N": N, "B": B, "vals": to_dev(torch, A["b_val"], cuda), "rp": to_dev(torch, A["b_row_ptr"].astype(np.int32), cuda),
+             "ci": to_dev(torch, A["b_col_idx"].astype(np.int32), cuda), "Bd": to_dev(torch, B, cuda)}
+        t["C"] = torch.full((A["M"], N), 0x7E00, dtype=torch.int16, device=cuda)
+        return t
+
+    def drop_in(t):
+        A = t["A"]
+        t["C"].fill_(0x7E00)
+        smat.spmm(t["vals"], t["rp"], t["ci"], t["Bd"], t["C"], A["M"], t["N"], A["K"], A["nnzb"], drop_in=True)
+        torch.cuda.synchronize()
+        return t["C"].cpu().numpy().view(np.uint16)
+
+    def planned(t):
+        A = t["A"]
+        p = smat.Plan(A["b_row_ptr"], A["M"], A["K"], A["nnzb"], t["N"], col_idx_host=A["b_col_idx"])
+        kernel = p.info()["kernel"]
+        Cp = torch.full((A["M"], t["N"]), 0x7E00, dtype=torch.int16, device=cuda)
+        smat.spmm(t["vals"], t["rp"], t["ci"], t["Bd"], Cp, A["M"], t["N"], A["K"], A["nnzb"], plan=p)
+        torch.cuda.synchronize()
+        p.close()
+        return Cp.cpu().numpy().view(np.uint16), kernel
+
+    one = setup(gen.random_bcsr(512, 64, 0.2, seed=31), 2048, 41)   # the plan's choice is the sweep kernel
+    two = setup(gen.random_bcsr(96, 80, 0.2, seed=32), 264, 42)     # row-wise
+    want1, k1 = planned(one)
+    want2, k2 = planned(two)
+    assert (k1, k2) == (SWEEP, 1)
+    s0 = cache_stats(smat)
+    for t, want in ((one, want1), (two, want2), (one, want1), (two, want2), (two, want2)):
+        assert np.array_equal(drop_in(t), want)
+    s1 = cache_stats(smat)
+    assert s1["built"] - s0["built"] == 2 and s1["hits"] - s0["hits"] == 3 and s1["entries"] == 2
+    assert oracle.compare(want1, oracle_ref(oracle, one["A"], one["B"], one["N"]))[0] <= TOL_F16
+    # block values are read by every launch: new values in the same array, same plan, new result
+    one["vals"].copy_(to_dev(torch, gen.random_bcsr(512, 64, 0.2, seed=31)["b_val"][::-1].copy(), cuda))
+    A1b = dict(one["A"], b_val=one["A"]["b_val"][::-1].copy())
+    assert oracle.compare(drop_in(one), oracle_ref(oracle, A1b, one["B"], one["N"]))[0] <= TOL_F16
+    assert cache_stats(smat)["built"] == s1["built"]
+    # another block pattern written into the same arrays (same number of blocks): the checksum, taken on every
+    # call here instead of every 64th, sees it and the plan is made again
+    other = gen.random_bcsr(96, 80, 0.0, seed=33, row_lengths=np.diff(two["A"]["b_row_ptr"])[::-1].tolist())
+    assert other["nnzb"] == two["A"]["nnzb"] and not np.array_equal(other["b_col_idx"], two["A"]["b_col_idx"])
+    two["rp"].copy_(to_dev(torch, other["b_row_ptr"].astype(np.int32), cuda))
+    two["ci"].copy_(to_dev(torch, other["b_col_idx"].astype(np.int32), cuda))
+    two["vals"].copy_(to_dev(torch, other["b_val"], cuda))
+    two["A"] = other
+    lib.smat_internal_plan_cache_check_every(C.c_uint64(1))
+    got = drop_in(two)
+    lib.smat_internal_plan_cache_check_every(C.c_uint64(0))
+    assert cache_stats(smat)["rebuilt"] == s1["rebuilt"] + 1
+    assert oracle.compare(got, oracle_ref(oracle, other, two["B"], two["N"]))[0] <= TOL_F16
+    # the explicit way: clear the cache
+    assert lib.smat_plan_cache_clear() == 0 and cache_stats(smat)["entries"] == 0
+    # switched off: plain launches of the row-wise kernel, nothing kept
+    monkeypatch.setenv("SMAT_PLAN_CACHE", "0")
+    b = cache_stats(smat)["built"]
+    assert oracle.compare(drop_in(two), oracle_ref(oracle, other, two["B"], two["N"]))[0] <= TOL_F16
+    assert cache_stats(smat)["built"] == b and cache_stats(smat)["entries"] == 0
+    monkeypatch.delenv("SMAT_PLAN_CACHE")
+    # with SMAT_PLAN_CACHE=values the cached plan looks at the values too: a matrix with about one nonzero per block
+    # goes through the compact kernel, the same bits as an explicit plan with attached values
+    monkeypatch.setenv("SMAT_PLAN_CACHE", "values")
+    d = gen.erdos_renyi(2048, 0.004)
+    sp = setup(bcsr_of(smat, d), 128, 43)
+    Cc, info = gpu_spmm_compact(smat, cuda, sp["A"], sp["B"], 128, kernel=0)
+    assert info["kernel"] == COMPACT
+    assert np.array_equal(drop_in(sp), Cc)
+    lib.smat_plan_cache_clear()
 
 
 def test_empty_matrix_and_empty_rows_write_zeros(smat, cuda, oracle):

@@ -12,8 +12,10 @@ import bench
 
 HERE = os.path.dirname(os.path.abspath(__file__))
 GOLDEN = json.load(open(os.path.join(HERE, "golden", "structure_hashes.json")))
-# the reordered R-MAT scale 20 workload needs a ten-minute reorder: its entry is checked by bench.py --perm-file
+# the reordered R-MAT scale 20 workload (permutations from tests/golden/rmat_s20_deg16_perms.npz) takes minutes to
+# build on few cores: it runs with the GPU tests only, here and in tests/test_gpu_full_size.py
 NAMES = [n for n in sorted(GOLDEN) if n != "rmat_s20_deg16_reordered_N128"]
+REFERENCE_DERIVED = [n for n in sorted(GOLDEN) if "reference" in GOLDEN[n]]
 
 
 def check(name):
@@ -27,12 +29,23 @@ def check(name):
         assert bench.INFO["perm_sha256"] == want["perm_sha256"]
     res = bench.structure_against_golden(name, A)
     assert res is not None and res["ok"] and not res["differs"]
+    if "reference" in want:
+        # the reference's own program, run on this pattern and then on the transpose of its output, ends with the
+        # same blocked structure and reports the same counters (comparisons, merges, blocks, longest row) per pass
+        ref = want["reference"]
+        assert res["equals_reference_program"]
+        assert want["pattern_sha256"] == ref["pattern_sha256"] and want["nnzb"] == ref["nnzb"]
+        assert bench.INFO["reorder_counters"] == [ref["stats_rows"], ref["stats_cols"]]
     return A
 
 
 def test_fixture_covers_every_config():
     assert len(GOLDEN) >= 9 and "rmat_s20_deg16_reordered_N128" in GOLDEN
     assert all(len(e["pattern_sha256"]) == 64 for e in GOLDEN.values())
+    # the reordered forms of configs 2 and 5 at full size and of config 3 at reduced scales are pinned to the
+    # output of the reference's reorder program
+    assert {"er_16384_0.1pct_reordered_N256", "stencil27_64_reordered_N64", "rmat_s15_deg16_reordered_N128",
+            "rmat_s16_deg16_reordered_N128"} <= set(REFERENCE_DERIVED)
 
 
 @pytest.mark.parametrize("name", NAMES)
@@ -49,6 +62,7 @@ def test_a_changed_structure_is_reported():
 
 
 @pytest.mark.gpu
+@pytest.mark.timeout(900)
 @pytest.mark.parametrize("name", NAMES)
 def test_structure_on_the_gpu_machine(smat, cuda, name):
     check(name)

@@ -45,6 +45,12 @@ def run_both(smat, cuda, A, B_bits, N):
     torch.cuda.synchronize()
     after_plan = alloc_counts()
     assert after_plan[0] > counts_before_plan[0], "the counters do not see the plan's allocations"
+    # the first call on a device loads the kernels' code and looks up the fixed array (both the runtime's doing,
+    # once per process): the free memory is read after it
+    check(lib.smat_spmm_bcsr_f16_static(vals.data_ptr(), rp.data_ptr(), ci.data_ptr(), Bd.data_ptr(), C_new.data_ptr(),
+                                        M, N, K, nnzb, None))
+    torch.cuda.synchronize()
+    assert alloc_counts() == after_plan, "smat_spmm_bcsr_f16_static allocated or released device memory"
     free_before = torch.cuda.mem_get_info()[0]
     for _ in range(3):
         check(lib.smat_spmm_bcsr_f16_static(vals.data_ptr(), rp.data_ptr(), ci.data_ptr(), Bd.data_ptr(), C_new.data_ptr(),
