@@ -282,6 +282,7 @@ def main():
     ap.add_argument("--kernel", type=int, default=0, help="0 auto, 1 rowwise, 2 sweep, 3 rowwise reading B in place, 5 compact, 6 mixed (rowwise + compact by block row)")
     ap.add_argument("--no-plan", action="store_true")
     ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--no-static-mix", action="store_true", help="skip the static-schedule micro-benchmark that the sweep kernel is compared with")
     ap.add_argument("--no-verify", action="store_true", help="skip the check of sampled block rows against the CPU oracle")
     ap.add_argument("--no-attach-values", action="store_true",
                     help="do not let the plan look at the block values (the compact kernel, id 5, needs them)")
@@ -410,6 +411,17 @@ def main():
     roof["measured_mfma_peak_tflops"] = round(peak.value, 1)
     if mfma_bound and peak.value > 0:
         roof["frac_of_measured_mfma_peak"] = round(ach_tflops / peak.value, 4)
+    if kernel_id == 2 and not args.no_static_mix:
+        # what the sweep kernel's data flow delivers on a static schedule (smat_bench_static_mix), on this device, now
+        mix = {}
+        for key, variant in (("lds_reads_and_mfma", 0), ("full_mix_a_in_l2", 1), ("full_mix", 2),
+                             ("full_mix_a_in_l2_barrier_per_8_ops", 3), ("full_mix_barrier_per_8_ops", 4)):
+            t = C.c_double()
+            check(lib.smat_bench_static_mix(variant, C.byref(t)))
+            mix[key] = round(t.value, 1)
+        roof["static_mix_tflops"] = mix["full_mix"]
+        roof["frac_of_static_mix"] = round(ach_tflops / mix["full_mix"], 4) if mix["full_mix"] > 0 else None
+        roof["static_mix_variants_tflops"] = mix
     roof["algorithmic_flops"] = flops
     roof["algorithmic_bytes"] = qbytes
     roof["hbm_gbs_at_algorithmic_bytes"] = round(ach_gbs, 1)

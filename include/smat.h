@@ -325,6 +325,14 @@ int smat_event_elapsed_ms(void *start, void *stop, float *ms);
  * nothing but v_mfma_f32_16x16x32_f16 on registers, in TFLOP/s (best of seven timed passes, about 1 ms each).
  * The published peak assumes the maximum clock; this is what the card sustains. */
 int smat_bench_mfma_peak(double *tflops);
+/* Benchmark helper (no counterpart in the reference): the rate, in TFLOP/s of its MFMAs, of a kernel with the sweep
+ * kernel's geometry and steady-state instruction mix on a static, regular schedule (8 wavefronts per CU; per op 4 LDS
+ * reads of 1 KiB, one 1 KiB load of A, 5/8 of a 1 KiB global->LDS copy, 4 MFMAs), i.e. what the data flow delivers
+ * without any bookkeeping.  variant 0: LDS reads and MFMAs only; 1: the full mix with the A operands inside 1 MiB
+ * (resident in the L2); 2: the full mix with A spread over 13 MB like the headline matrix, the 8 workgroups of an
+ * XCD slot reading the same blocks; 3 and 4: variants 1 and 2 with a workgroup barrier every 8 ops.  Best of four
+ * timed passes of about a millisecond. */
+int smat_bench_static_mix(int variant, double *tflops);
 
 #ifdef __cplusplus
 }

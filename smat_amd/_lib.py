@@ -77,6 +77,7 @@ SIGNATURES = {
     "smat_event_synchronize": (_int, [_vp]),
     "smat_event_elapsed_ms": (_int, [_vp, _vp, C.POINTER(C.c_float)]),
     "smat_bench_mfma_peak": (_int, [C.POINTER(C.c_double)]),
+    "smat_bench_static_mix": (_int, [_int, C.POINTER(C.c_double)]),
 }
 
 

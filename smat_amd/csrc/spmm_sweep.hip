@@ -45,6 +45,7 @@ namespace smat {
 typedef _Float16 f16x8 __attribute__((ext_vector_type(8)));
 typedef float f32x4 __attribute__((ext_vector_type(4)));
 typedef int i32x4 __attribute__((ext_vector_type(4)));
+typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
 
 namespace {
 
@@ -236,8 +237,23 @@ __global__ __launch_bounds__(THREADS) void spmm_sweep_kernel(
                               (_Float16)v1[0], (_Float16)v1[1], (_Float16)v1[2], (_Float16)v1[3]};
             const f16x8 h1 = {(_Float16)v2[0], (_Float16)v2[1], (_Float16)v2[2], (_Float16)v2[3],
                               (_Float16)v3[0], (_Float16)v3[1], (_Float16)v3[2], (_Float16)v3[3]};
-            if (nbase < N) *reinterpret_cast<f16x8 *>(crow) = h0;
-            if (nbase + 8 < N) *reinterpret_cast<f16x8 *>(crow + 8) = h1;
+            // h0 / h1 are columns 16g .. 16g+7 / 16g+8 .. 16g+15 of this lane's row.  Stored as they are, one store
+            // instruction would write four 16-byte pieces with 16-byte holes into every 128-byte row.  Two lane
+            // swaps (rows of 16 lanes, then halves of the wavefront) regroup them so that the first store writes
+            // bytes 0 .. 63 of each row and the second bytes 64 .. 127, 16 bytes per lane at 16 * g.
+            (void)crow;
+            const u32x4 x = __builtin_bit_cast(u32x4, h0), y = __builtin_bit_cast(u32x4, h1);
+            u32x4 d1, d2;
+#pragma unroll
+            for (int w = 0; w < 4; w++) {
+                const auto r = __builtin_amdgcn_permlane16_swap(x[w], y[w], false, false); // {X0 Y0 X2 Y2}, {X1 Y1 X3 Y3} by lane row
+                const auto q = __builtin_amdgcn_permlane32_swap(r[0], r[1], false, false); // {X0 Y0 X1 Y1}, {X2 Y2 X3 Y3}
+                d1[w] = q[0];
+                d2[w] = q[1];
+            }
+            uint16_t *row0 = reinterpret_cast<uint16_t *>(Cout) + m * (long)N + n0 + 8 * g;
+            if (n0 + 8 * g < N) *reinterpret_cast<u32x4 *>(row0) = d1;
+            if (n0 + 32 + 8 * g < N) *reinterpret_cast<u32x4 *>(row0 + 32) = d2;
         }
     };
     store_row(std::integral_constant<int, 0>{}); store_row(std::integral_constant<int, 1>{});
