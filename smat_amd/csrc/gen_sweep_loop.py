@@ -7,7 +7,7 @@ to the block of the next descriptor.  A block is specialised for
 
     J  the position of the op in the stream modulo 8 (which register sets it uses),
     r  the block row of the wavefront the op adds to (which accumulators),
-    v  whether copies were issued between the load of its A operand and now (which s_waitcnt vmcnt),
+    v  whether the copies of a chunk boundary were issued between the load of its A operand and now (which s_waitcnt vmcnt),
 
 so the run-time choices cost no instruction besides the jump.  It is written by hand because a
 wavefront issues in order: every instruction next to its MFMAs adds to its run time.  Blocks have a
@@ -28,16 +28,18 @@ Stream position i, J = i % 8.  Block of op i (AHEAD = 4):
     The set that the reads of op i + 1 land in is the one the MFMAs of op i - 1 took their operands from a few
     instructions earlier: an MFMA reads its A and B sources when it starts, LDS data arrives 64 clocks later
     at the earliest.
-Marker (first thing of every chunk but the first): own copies of the next chunk have landed, barrier,
-copies of the chunk after next, and the same read-ahead duties, no MFMAs.
+Chunk boundary (before the first op of every chunk but the first): the descriptor of that op names a trampoline
+instead of its block; the trampoline notes the block's offset and branches to the boundary code: own copies of
+the next chunk have landed, barrier, copies of the chunk after next, then on to the op's block.  The boundary is
+no stream position: no operand load and no descriptor slot is spent on it.
 
 Registers (fixed, all listed as clobbers):
     v40-v71    B operands, two sets of 4 tiles x 4 registers
     v72-v103   A operands, ring of eight
     v104-v106  temporaries
     s40-s71    descriptor ring, op i in slot i % 8: w0 w1 w2 w3
-    s72-s85    state: descriptor pointer, code base, chunk counter, next chunk id, chunk list pointer,
-               temporaries, jump target
+    s72-s86    state: descriptor pointer, code base, chunk counter, next chunk id, chunk list pointer,
+               temporaries, jump target, the block a chunk boundary continues with
     a0-a127    accumulators (block row r, tile t in a[16r + 4t .. + 3])
 """
 
@@ -51,17 +53,21 @@ BSETS, ARING = 2, 8                      # B operands are read from LDS one posi
 
 RING = 8
 BLOCK_BYTES = 128                        # SWEEP_BLOCK_BYTES
-MARK_BASE = 8 * 8 * 2 * BLOCK_BYTES      # SWEEP_MARK_BASE: after the 128 op blocks
+N_BLOCKS = 8 * 8 * 2                     # SWEEP_N_BLOCKS: stream position % 8 x block row x v
+TRAMP_BASE = N_BLOCKS * BLOCK_BYTES      # SWEEP_TRAMP_BASE: after the op blocks
+TRAMP_BYTES = 8                          # SWEEP_TRAMP_BYTES
+MARK_OFF = TRAMP_BASE + N_BLOCKS * TRAMP_BYTES   # SWEEP_MARK_OFF
 MARK_BYTES = 512                         # SWEEP_MARK_BYTES
-END_OFF = MARK_BASE + 8 * MARK_BYTES     # SWEEP_END_OFF
+END_OFF = MARK_OFF + MARK_BYTES          # SWEEP_END_OFF
 COPIES = 4
-MIN_OPS = max(AHEAD - 1, COPIES)
-VM_MARK = MIN_OPS + 1      # a marker's copies of one marker ago are older than the A loads of the MIN_OPS + 1 positions since
+MIN_OPS = AHEAD            # SWEEP_MIN_OPS
+VM_MARK = MIN_OPS          # a boundary's copies of one boundary ago are older than the A loads of the MIN_OPS positions since
 
 S_RING0 = 40
 DESC_AHEAD = 7   # an odd position loads the descriptors of ops i + DESC_AHEAD and the one after
 S_DP, S_BASE, S_CUR, S_NEXTK, S_CP, S_T0, S_T1, S_JMP = 72, 74, 76, 77, 78, 80, 81, 84
-S_LAST = 85
+S_RET = 86
+S_LAST = 86
 V_B0 = 40
 V_A0 = V_B0 + 16 * BSETS
 V_T0 = V_A0 + 4 * ARING
@@ -142,16 +148,22 @@ def op_block(J, r, v):
     emit(f".org Lb0_%= + {(k + 1) * BLOCK_BYTES}")
 
 
-def marker_block(J):
-    label(f"Lm{J}")
-    top_wait(J)                                       # the reads of the ops of the chunk that ends here are in registers
-    emit(f"s_waitcnt vmcnt({VM_MARK})")               # own copies of the chunk after the one being entered (issued one marker ago) have landed
+def trampoline(k):
+    label(f"Lt{k}")
+    emit(f"s_movk_i32 s{S_RET}, {k * BLOCK_BYTES}")
+    emit("s_branch Lmark_%=")
+    emit(f".org Lb0_%= + {TRAMP_BASE + (k + 1) * TRAMP_BYTES}")
+
+
+def boundary_code():
+    label("Lmark")
+    emit(f"s_waitcnt vmcnt({VM_MARK})")               # own copies of the chunk after the one being entered (issued one boundary ago) have landed
     emit("s_barrier")
     emit(f"s_add_u32 s{S_CUR}, s{S_CUR}, 1")          # chunk (position in the row group's list) being entered
     emit(f"s_add_u32 s{S_T0}, s{S_CUR}, 2")
     emit(f"s_cmp_ge_u32 s{S_T0}, %[n_chunks]")
-    emit(f"s_cbranch_scc1 Lmn{J}_%=")
-    # copies of chunk cur + 2 into stage (cur + 2) % 4: rows of B from k = 256 * id (the id was loaded by the previous marker)
+    emit("s_cbranch_scc1 Lmn_%=")
+    # copies of chunk cur + 2 into stage (cur + 2) % 4: rows of B from k = 256 * id (the id was loaded by the previous boundary)
     emit(f"s_lshl_b32 s{S_T1}, s{S_NEXTK}, 9")
     emit(f"v_add_u32 v{V_COPY}, s{S_T1}, %[copy_off]")
     emit(f"v_min_u32 v{V_COPY}, v{V_COPY}, %[copy_lim]")
@@ -162,13 +174,14 @@ def marker_block(J):
         emit(f"s_add_u32 m0, s{S_T0}, {1024 * it}")
         emit("s_nop 0")
         emit(f"global_load_lds_dwordx4 v{V_COPY}, %[sb{it}]")
-    label(f"Lmn{J}")
-    emit(f"s_load_dword s{S_NEXTK}, s[{S_CP}:{S_CP + 1}], 0x0")   # id of chunk cur + 3, for the next marker
+    label("Lmn")
+    emit(f"s_load_dword s{S_NEXTK}, s[{S_CP}:{S_CP + 1}], 0x0")   # id of chunk cur + 3, for the next boundary
     emit(f"s_add_u32 s{S_CP}, s{S_CP}, 4")
     emit(f"s_addc_u32 s{S_CP + 1}, s{S_CP + 1}, 0")
-    a_load(J + AHEAD)
-    jump(J + 1)
-    emit(f".org Lb0_%= + {MARK_BASE + (J + 1) * MARK_BYTES}")
+    emit(f"s_add_u32 s{S_JMP}, s{S_BASE}, s{S_RET}")             # on to the block of the op that opens the chunk
+    emit(f"s_addc_u32 s{S_JMP + 1}, s{S_BASE + 1}, 0")
+    emit(f"s_setpc_b64 s[{S_JMP}:{S_JMP + 1}]")
+    emit(f".org Lb0_%= + {MARK_OFF + MARK_BYTES}")
 
 
 # ---- entry: descriptors of ops 0..5, A operands of ops 0..AHEAD-1, B operands of ops 0 and 1 ----
@@ -200,16 +213,17 @@ for J in range(8):
     for r in range(8):
         for v in range(2):
             op_block(J, r, v)
-for J in range(8):
-    marker_block(J)
+for k in range(N_BLOCKS):
+    trampoline(k)
+boundary_code()
 label("Lend")                                         # offset END_OFF: the descriptor after the last op jumps here
 emit("s_waitcnt vmcnt(0) lgkmcnt(0)")
 
 clob = ([f'"v{i}"' for i in range(V_B0, V_COPY + 1)] + [f'"s{i}"' for i in range(S_RING0, S_LAST + 2)] +
         [f'"a{i}"' for i in range(128)] + ['"vcc"', '"scc"', '"memory"'])
 print("// generated by gen_sweep_loop.py; do not edit")
-print(f"static_assert(SWEEP_AHEAD == {AHEAD} && SWEEP_BLOCK_BYTES == {BLOCK_BYTES} && SWEEP_MARK_BASE == {MARK_BASE} && "
-      f"SWEEP_MARK_BYTES == {MARK_BYTES} && SWEEP_END_OFF == {END_OFF}, \"regenerate spmm_sweep_loop.inc\");")
+print(f"static_assert(SWEEP_AHEAD == {AHEAD} && SWEEP_MIN_OPS == {MIN_OPS} && SWEEP_BLOCK_BYTES == {BLOCK_BYTES} && SWEEP_TRAMP_BASE == {TRAMP_BASE} && "
+      f"SWEEP_TRAMP_BYTES == {TRAMP_BYTES} && SWEEP_MARK_OFF == {MARK_OFF} && SWEEP_END_OFF == {END_OFF}, \"regenerate spmm_sweep_loop.inc\");")
 print("asm volatile(")
 for line in out:
     end = "\\n" if line.endswith(":") else "\\n\\t"

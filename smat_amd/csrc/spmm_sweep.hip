@@ -23,13 +23,14 @@
 //  * Pipeline.  The B operands of an op are read from LDS one position ahead (two register sets), its A
 //    operand (two neighbouring 512-byte blocks, one load straight into MFMA layout) comes from global memory
 //    four positions ahead (ring of eight).  Vector memory operations complete in order, so the number of
-//    younger ones at every wait is known when the plan is built: 4, or 8 when a marker issued its copies in
+//    younger ones at every wait is known when the plan is built: 4, or 8 when a chunk boundary issued its copies in
 //    between.  A half of an MFMA that must not contribute (unpaired block) reads a 16 KiB region of zeros.
 //  * Accumulators live in a[0:127] and are touched by inline assembly only.
-//  * Synchronisation.  One barrier per chunk, in the marker entry that starts the chunk.  Marker of chunk c:
-//    the wavefront's own copies of chunk c+1 (issued one marker earlier) have landed, barrier, then the copies
-//    of chunk c+2 go into the stage that held chunk c-2.  The plan gives every wavefront at least four ops
-//    per chunk (filler ops that multiply zeros where it has fewer), so markers are at least five positions
+//  * Synchronisation.  One barrier per chunk, in the boundary code that the first op of the chunk runs through
+//    before its own block (it is no stream position: no descriptor, no operand load is spent on it).  Boundary of
+//    chunk c: the wavefront's own copies of chunk c+1 (issued one boundary earlier) have landed, barrier, then the
+//    copies of chunk c+2 go into the stage that held chunk c-2.  The plan gives every wavefront at least four ops
+//    per chunk (filler ops that multiply zeros where it has fewer), so boundaries are at least four positions
 //    apart and every wavefront passes every barrier.
 //
 // Same operand semantics as the reference launcher (src/cuda_hgemm/src/mma/mmaCBT.cu:83-88).

@@ -16,7 +16,7 @@ namespace smat {
 namespace {
 constexpr int G = SWEEP_G, RW = SWEEP_RW, WAVES = SWEEP_WAVES, S = SWEEP_S, MIN_OPS = SWEEP_MIN_OPS;
 constexpr int AHEAD = SWEEP_AHEAD, COPIES = SWEEP_COPIES;
-constexpr int VM_MARK = MIN_OPS + 1; // a marker waits until at most this many vector memory operations are under way
+constexpr int VM_MARK = MIN_OPS; // a chunk boundary waits until at most this many vector memory operations are under way
 } // namespace
 
 void build_sweep_plan(const int32_t *row_ptr, const int32_t *col_idx, size_t mb, size_t kb, SweepPlanHost &out,
@@ -223,18 +223,18 @@ void build_sweep_plan(const int32_t *row_ptr, const int32_t *col_idx, size_t mb,
             if (left) throw std::logic_error("sweep plan: ops left over by the period schedule");
         }
 
-        // ---- streams: ops of chunk 0, marker, ops of chunk 1, ..., end ----
+        // ---- streams: ops of chunk 0, ops of chunk 1, ..., end; the first op of a chunk carries the chunk boundary ----
         for (int w = 0; w < WAVES; w++) {
             out.op_ptr.push_back((int32_t)out.ops.size());
             if (n_chunks == 0) continue; // the kernel does not enter the interpreter for an empty row group
             by_chunk = schedule[(size_t)w];
-            struct Item { int kind, row; SweepOpHost op; }; // kind: 0 op, 1 marker, 2 end
+            struct Item { int kind, row; bool opens; SweepOpHost op; }; // kind: 0 op, 2 end; opens: first op of a chunk but the first
             std::vector<Item> items;
-            const SweepOpHost idle{0, SWEEP_ZERO_OFF, 0, 0}; // markers and the end: no blocks of their own
+            const SweepOpHost idle{0, SWEEP_ZERO_OFF, 0, 0}; // the end: no blocks of its own
             // A filler op multiplies two blocks by zeros and adds the result to one of the wavefront's block rows:
             // two blocks of that very row (then an Inf or NaN in them is in that row of C anyway), blocks 0 and 1
             // of the matrix only when no row of the wavefront has two.
-            Item filler{0, 0, idle};
+            Item filler{0, 0, false, idle};
             for (int r = 0; r < RW; r++) {
                 const int32_t br = out.row_map[(rg * WAVES + (size_t)w) * RW + (size_t)r];
                 if (br >= 0 && row_ptr[br + 1] - row_ptr[br] >= 2) {
@@ -249,28 +249,33 @@ void build_sweep_plan(const int32_t *row_ptr, const int32_t *col_idx, size_t mb,
                     if (a.rank != b.rank) return a.rank < b.rank;
                     return a.row < b.row;
                 });
+                const size_t first_of_chunk = items.size();
+                size_t n_here = list.size();
                 if (c > 0) {
-                    items.push_back(Item{1, 0, idle});
-                    // The LDS reads of the first op after a marker are issued before the marker's barrier, when the
-                    // copies of chunk c + 1 may still be under way: that op has to be one whose chunks are c or c - 1.
+                    // The LDS reads of the op that opens a chunk are issued by the op before it, before the barrier of
+                    // the boundary, when the copies of chunk c + 1 may still be under way: it has to be an op whose
+                    // chunks are c or c - 1.
                     size_t ok = 0;
                     while (ok < list.size() && list[ok].hi > (int32_t)c) ok++;
                     if (ok == list.size()) {
                         items.push_back(filler);
                         out.n_fillers++;
+                        n_here++;
                     } else if (ok > 0) {
                         std::rotate(list.begin(), list.begin() + (long)ok, list.begin() + (long)ok + 1);
                     }
                 }
-                for (const Ranked &x : list) items.push_back(Item{0, x.row, x.op});
-                for (size_t k = list.size(); k < (size_t)MIN_OPS; k++) { // filler ops keep the markers AHEAD positions apart
+                for (const Ranked &x : list) items.push_back(Item{0, x.row, false, x.op});
+                for (size_t k = n_here; k < (size_t)MIN_OPS; k++) { // filler ops keep the chunk boundaries AHEAD positions apart
                     items.push_back(filler);
                     out.n_fillers++;
                 }
+                if (c > 0) items[first_of_chunk].opens = true;
             }
-            items.push_back(Item{2, 0, idle});
+            items.push_back(Item{2, 0, false, idle});
             // Which s_waitcnt vmcnt an op needs: vector memory operations complete in order, every position issues
-            // one A load (for the op AHEAD positions later), a marker issues its copies before that load.
+            // one A load (for the op AHEAD positions later), the op that opens a chunk issues the copies of the
+            // boundary before that load.
             std::vector<long> a_issue(items.size() + (size_t)AHEAD + 1, 0), copy_seq(n_chunks + 3, 0);
             long seq = 0;
             for (int k = 0; k < AHEAD; k++) a_issue[(size_t)k] = ++seq; // entry code, after the copies of chunks 0..2
@@ -281,23 +286,23 @@ void build_sweep_plan(const int32_t *row_ptr, const int32_t *col_idx, size_t mb,
                     it.op.w3 = SWEEP_END_OFF;
                     break;
                 }
-                if (it.kind == 1) {
+                if (it.opens) {
                     cur++;
-                    // the copies of chunk cur + 1 were issued by the marker before this one (or by the entry code)
-                    if (cur + 1 < n_chunks && seq - copy_seq[cur + 1] < VM_MARK) throw std::logic_error("sweep plan: a marker would not wait for its copies");
+                    // the copies of chunk cur + 1 were issued by the boundary before this one (or by the entry code): the
+                    // boundary waits until at most VM_MARK younger operations are under way
+                    if (cur + 1 < n_chunks && seq - copy_seq[cur + 1] < VM_MARK) throw std::logic_error("sweep plan: a chunk boundary would not wait for its copies");
                     if (cur + 2 < n_chunks) {
                         seq += COPIES;
                         copy_seq[cur + 2] = seq;
                     }
-                    it.op.w3 = sweep_marker_code((int)i);
                 }
                 a_issue[i + (size_t)AHEAD] = ++seq;
-                if (it.kind == 0) {
-                    const long younger = seq - a_issue[i];
-                    if (younger != AHEAD && younger != AHEAD + COPIES) throw std::logic_error("sweep plan: markers closer than the A read-ahead");
-                    it.op.w3 = sweep_op_code((int)i, it.row, younger == AHEAD ? 0 : 1);
-                }
+                const long younger = seq - a_issue[i];
+                if (younger != AHEAD && younger != AHEAD + COPIES) throw std::logic_error("sweep plan: chunk boundaries closer than the A read-ahead");
+                const int v = younger == AHEAD ? 0 : 1;
+                it.op.w3 = it.opens ? sweep_boundary_op_code((int)i, it.row, v) : sweep_op_code((int)i, it.row, v);
             }
+            if (cur + 1 != n_chunks) throw std::logic_error("sweep plan: a stream does not pass every chunk boundary");
             for (const Item &it : items) out.ops.push_back(it.op);
         }
         for (size_t c = first_chunk; c < out.chunk_ids.size(); c++) local[(size_t)out.chunk_ids[c]] = -1;
@@ -312,7 +317,7 @@ void build_sweep_plan(const int32_t *row_ptr, const int32_t *col_idx, size_t mb,
 
 // Test hook (not part of smat.h): builds the work list on the host (rows != NULL: of these block rows only) and hands it out.  Arrays are
 // allocated with malloc; release each with smat_host_free.  row_map: n_rg * 64 block rows (-1 = none).  counts[0..5] = row groups, listed
-// chunks, stream entries (ops, fillers, markers, ends; without padding), pairs, singles, fillers.
+// chunks, stream entries (ops, fillers, ends; without padding), pairs, singles, fillers.
 static int smat_internal_sweep_plan_impl(const int32_t *row_ptr, const int32_t *col_idx, size_t M, size_t K,
                                          const int32_t *rows, size_t n_rows, int32_t **rg_chunk_ptr, int32_t **chunk_ids, int32_t **op_ptr,
                                          uint32_t **ops, int32_t **row_map, int64_t *counts)
@@ -345,7 +350,7 @@ static int smat_internal_sweep_plan_impl(const int32_t *row_ptr, const int32_t *
     return SMAT_OK;
 }
 
-// Test hook: the pipeline depths this build was compiled with {A read-ahead, LDS read-ahead, minimum ops per chunk, copies per marker}.
+// Test hook: the pipeline depths this build was compiled with {A read-ahead, LDS read-ahead, minimum ops per chunk, copies per chunk boundary}.
 extern "C" void smat_internal_sweep_params(int32_t *out)
 {
     out[0] = smat::SWEEP_AHEAD; out[1] = smat::SWEEP_LDS_AHEAD; out[2] = smat::SWEEP_MIN_OPS; out[3] = smat::SWEEP_COPIES;

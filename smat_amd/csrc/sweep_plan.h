@@ -18,7 +18,7 @@ struct SweepPlanHost {
     std::vector<int32_t> chunk_ids;    // K chunk of every (row group, listed chunk), + SWEEP_CHUNK_PAD entries
     std::vector<int32_t> op_ptr;       // n_rg * 8 + 1
     std::vector<int32_t> row_map;      // n_rg * 64: block row of (row group, wavefront, local row), -1 = none
-    std::vector<SweepOpHost> ops;      // streams (ops, markers, ends) + SWEEP_OP_PAD entries
+    std::vector<SweepOpHost> ops;      // streams (ops, ends) + SWEEP_OP_PAD entries
     size_t n_pairs = 0, n_singles = 0, n_fillers = 0;
 };
 

@@ -17,10 +17,12 @@ G, RW, WAVES, S, STAGES = 64, 8, 8, 16, 4
 _params = (C.c_int32 * 4)()
 lib.smat_internal_sweep_params(_params)
 AHEAD, PB, MIN_OPS, COPIES = (int(x) for x in _params)  # A read-ahead, LDS read-ahead (positions), ops per chunk, copies per marker
-assert (AHEAD, PB) in ((3, 2), (4, 1), (5, 1)) and MIN_OPS == max(AHEAD - 1, COPIES)
+assert (AHEAD, PB) == (4, 1) and MIN_OPS == AHEAD
 ZERO_OFF = 131072
-BLOCK_BYTES, MARK_BASE, MARK_BYTES = 128, 16384, 512
-END_OFF = MARK_BASE + 8 * MARK_BYTES
+BLOCK_BYTES, N_BLOCKS, TRAMP_BYTES = 128, 128, 8
+TRAMP_BASE = N_BLOCKS * BLOCK_BYTES         # first ops of a chunk go through a trampoline: chunk boundary code, then the op's block
+MARK_OFF = TRAMP_BASE + N_BLOCKS * TRAMP_BYTES
+END_OFF = MARK_OFF + 512
 LDS_MASK = 0x1C0E0
 PAD, CHUNK_PAD = 16, 4
 
@@ -57,9 +59,9 @@ def sweep_plan(row_ptr, col_idx, M, K, rows=None):
         load = np.zeros((WAVES, max(n_periods, 1)), int)
         for w in range(WAVES):
             w3 = plan["ops"][plan["op_ptr"][rg * WAVES + w]:plan["op_ptr"][rg * WAVES + w + 1], 3]
-            marks = (w3 >= MARK_BASE) & (w3 < END_OFF)
-            period = np.cumsum(marks)
-            is_op = w3 < MARK_BASE
+            opens = (w3 >= TRAMP_BASE) & (w3 < MARK_OFF)
+            period = np.cumsum(opens)
+            is_op = w3 < MARK_OFF
             np.add.at(load[w], period[is_op], 1)
         total += int(load.max(0).sum())
     plan["period_max_sum"] = total
@@ -96,41 +98,42 @@ def replay(plan, A, Bd, rows=None):
                 assert ops.shape[0] == 0
                 continue
             # vector memory operations in issue order: the entry code loads the A operands of positions 0..AHEAD-1 after
-            # the copies of chunks 0..2; position i loads the operand of i + AHEAD, a marker issues its copies first
+            # the copies of chunks 0..2; position i loads the operand of i + AHEAD, an op that opens a chunk issues the
+            # copies of the chunk boundary first
             seq = AHEAD
             a_issue = {k: k + 1 for k in range(AHEAD)}
             copy_seq = {0: 0, 1: 0, 2: 0}
             cur, in_chunk, ended = 0, 0, False
-            period = []  # chunk period of every stream position (a marker belongs to the chunk it opens)
+            period = []  # chunk period of every stream position
             for i, (w0, w1, w2, w3) in enumerate(tuple(int(x) for x in e) for e in ops):
                 assert not ended, "entries after the end of a stream"
-                # what the LDS reads issued at this position may see: a marker issues its reads behind its barrier when
-                # they are two positions ahead (it then belongs to the chunk it opens), before it when one ahead
-                period.append(cur + 1 if END_OFF > w3 >= MARK_BASE and PB == 2 else cur)
                 if w3 == END_OFF:
                     assert (w0, w1, w2) == (0, ZERO_OFF, 0)
                     ended = True
                     continue
-                if w3 >= MARK_BASE:
-                    assert (w3 - MARK_BASE) % MARK_BYTES == 0 and (w3 - MARK_BASE) // MARK_BYTES == i % 8
-                    assert (w0, w1, w2) == (0, ZERO_OFF, 0)
+                assert w3 < MARK_OFF, "an entry names code that is no op block and no trampoline"
+                if w3 >= TRAMP_BASE:  # chunk boundary in front of this op: own copies landed, barrier, next copies
+                    assert (w3 - TRAMP_BASE) % TRAMP_BYTES == 0
+                    k = (w3 - TRAMP_BASE) // TRAMP_BYTES
                     assert in_chunk >= MIN_OPS, "fewer ops in a chunk than the read-ahead needs"
                     cur, in_chunk = cur + 1, 0
-                    # the marker waits until at most MIN_OPS + 1 operations are under way: its copies of the next chunk
-                    # (issued by the marker before it, or by the entry code) are older than that
+                    # the boundary waits until at most MIN_OPS operations are under way: its copies of the next chunk
+                    # (issued by the boundary before it, or by the entry code) are older than that
                     if cur + 1 < chunks.size:
-                        assert seq - copy_seq[cur + 1] >= MIN_OPS + 1
+                        assert seq - copy_seq[cur + 1] >= MIN_OPS
                     if cur + 2 < chunks.size:
                         seq += COPIES
                         copy_seq[cur + 2] = seq
-                    seq += 1
-                    a_issue[i + AHEAD] = seq
-                    continue
+                    opened = True
+                else:
+                    assert w3 % BLOCK_BYTES == 0
+                    k = w3 // BLOCK_BYTES
+                    opened = False
+                # what the LDS reads issued for this position could see: they were issued one position earlier
+                period.append(cur)
                 seq += 1
                 a_issue[i + AHEAD] = seq
                 in_chunk += 1
-                assert w3 % BLOCK_BYTES == 0
-                k = w3 // BLOCK_BYTES
                 pos, r, v = k // 16, (k // 2) % 8, k % 2
                 assert pos == i % 8, "code block of another stream position"
                 assert seq - a_issue[i] == AHEAD + COPIES * v, "wait class does not match the operations issued since the A load"
@@ -161,7 +164,8 @@ def replay(plan, A, Bd, rows=None):
                     # while chunk cur is swept the stages hold chunks cur - 1, cur and cur + 1 (the fourth is being filled)
                     held = [p for p in (cur + 1, cur, cur - 1) if 0 <= p < chunks.size and p % STAGES == stage]
                     assert held, "op reads the stage that is being overwritten"
-                    # its LDS reads were issued PB positions earlier: that chunk period sees the chunks up to the next one
+                    # its LDS reads were issued one position earlier (for the op that opens a chunk: in front of the
+                    # barrier, in the period before): that period sees the chunks up to its next one
                     assert held[0] <= period[max(i - PB, 0)] + 1
                     blk = q + half
                     k0 = int(chunks[held[0]]) * S * 16 + slab * 16
@@ -260,7 +264,7 @@ def test_single_last_block_is_listed_as_second_half():
     A = {"M": 32, "K": 640, "b_row_ptr": rp, "b_col_idx": ci, "b_val": gen.f16_bits(np.ones(ci.size * 256)), "nnzb": ci.size}
     plan = sweep_plan(rp, ci, 32, 640)
     real = plan["ops"][:plan["n_entries"]]
-    lo_zero = real[(real[:, 1] == ZERO_OFF) & (real[:, 2] != 0)]  # first half reads zeros, second half a stage
+    lo_zero = real[(real[:, 1] == ZERO_OFF) & (real[:, 2] != 0) & (real[:, 3] < MARK_OFF)]  # first half reads zeros, second half a stage
     assert lo_zero.shape[0] == 1 and lo_zero[0, 0] == (ci.size - 2) * 512
     Cd = replay(plan, A, np.ones((640, 8)))
     assert np.allclose(Cd, dense_of(A) @ np.ones((640, 8)))
@@ -276,7 +280,7 @@ def test_headline_matrix_pairs_nearly_everything():
     # hardly more ops than the average one (1.23 x without that freedom)
     assert plan["period_max_sum"] * WAVES < 1.08 * (plan["pairs"] + plan["singles"] + plan["fillers"])
     per_wave = np.diff(plan["op_ptr"])
-    assert per_wave.min() >= 4 * 32 + 32 and per_wave.max() <= 72 * 32
+    assert per_wave.min() >= 4 * 32 + 1 and per_wave.max() <= 72 * 32
 
 
 def test_committed_interpreter_loop_is_what_the_generator_writes():
