@@ -522,6 +522,26 @@ static int smat_plan_attach_values_impl(smat_plan *p, const uint16_t *vals, cons
     const int64_t blocks_sparse = (int64_t)p->nnzb - blocks_dense;
     // both kinds of rows matter (a tenth of the blocks each): mixed dispatch.  Otherwise one kernel for everything.
     bool mixed = may_mix && blocks_dense * 10 >= (int64_t)p->nnzb && blocks_sparse * 10 >= (int64_t)p->nnzb;
+    // the dense rows through the sweep kernel when their row groups of 64 fill the device, else row-wise
+    size_t n_dense_rows = 0;
+    for (size_t i = 0; may_mix && i < mb; i++) n_dense_rows += dense[i] != 0;
+    const bool dense_sweep_possible = !p->col_idx_host.empty() && blocks_dense >= 2 && p->nnzb < ((size_t)1 << 23) &&
+                                      p->K < ((size_t)1 << 28) && sweep_fills_device(n_dense_rows, p->n_cap);
+    bool dense_packed = p->d_bpack != nullptr; // row-wise route: B repacked slab-major first?
+    if (mixed && !dense_sweep_possible && want != SMAT_KERNEL_MIXED) {
+        // Row-wise route for the dense rows: it has to beat the compact kernel on those very rows, launch and (when B
+        // is repacked for it) the extra pass over B included.  Rates as measured: the compact kernel and the row-wise
+        // kernel on B in place gather about 8 TB/s of operand bytes, the row-wise kernel on repacked B 20 TB/s; a
+        // pass over B moves 4*K*N bytes at 4 TB/s; a launch costs 3 us.  (27-point stencil on 64^3 after the reorder,
+        // N = 64: a sixth of the blocks sit in dense rows, 13 us of compact kernel against 20 us for the repack alone.)
+        const double dense_cols = (double)(c->n_cols_all - c->n_cols);
+        const double t_compact = dense_cols * (double)p->n_cap * 2.0 / 8e6;
+        const double gather = (double)blocks_dense * 16.0 * (double)p->n_cap * 2.0;
+        const double t_direct = gather / 7.6e6 + 3.0;
+        const double t_packed = gather / 20e6 + 6.0 + 4.0 * (double)p->K * (double)p->n_cap / 4e6;
+        dense_packed = t_packed < t_direct;
+        if (std::min(t_direct, t_packed) >= 0.8 * t_compact) mixed = false;
+    }
     if (want == SMAT_KERNEL_MIXED) mixed = true;
     if (may_mix && !mixed && blocks_dense > 0) { // the list left dense rows out: make it whole again
         compact_destroy(c);
@@ -539,12 +559,14 @@ static int smat_plan_attach_values_impl(smat_plan *p, const uint16_t *vals, cons
         return SMAT_OK;
     }
     if (!p->d_bt) e = dev_malloc(&p->d_bt, p->bt_bytes());
-    // the dense rows through the sweep kernel when their row groups of 64 fill the device, else row-wise
     std::vector<int32_t> dense_list;
     for (size_t i = 0; mixed && i < mb; i++)
         if (dense[i]) dense_list.push_back((int32_t)i);
-    const bool dense_sweep = mixed && !p->col_idx_host.empty() && blocks_dense >= 2 && p->nnzb < ((size_t)1 << 23) &&
-                             p->K < ((size_t)1 << 28) && sweep_fills_device(dense_list.size(), p->n_cap);
+    const bool dense_sweep = mixed && dense_sweep_possible;
+    if (mixed && !dense_sweep) { // the scratch for the repacked B follows the choice made for the dense rows
+        if (dense_packed && !p->d_bpack && e == hipSuccess) e = dev_malloc(&p->d_bpack, p->K * p->n_cap * sizeof(uint16_t));
+        if (!dense_packed && p->d_bpack && want == SMAT_KERNEL_AUTO) { (void)dev_free(p->d_bpack); p->d_bpack = nullptr; }
+    }
     if (e == hipSuccess && dense_sweep) {
         SweepPlanHost h;
         build_sweep_plan(row_ptr_host, p->col_idx_host.data(), mb, p->K / 16, h, dense_list.data(), dense_list.size());
