@@ -32,11 +32,10 @@ void build_sweep_plan(const int32_t *row_ptr, const int32_t *col_idx, size_t mb,
     out.op_ptr.reserve(n_rg * WAVES + 1);
     out.row_map.assign(n_rg * G, -1);
     std::vector<int32_t> local(n_kchunks, -1); // K chunk -> position in the row group's chunk list
-    struct RowOp { int32_t exec, first, last, hi; SweepOpHost op; }; // nominal chunk period, the periods it may run in, its later chunk
+    struct RowOp { int32_t first, last, hi; SweepOpHost op; }; // the periods it may run in, its later chunk
     std::vector<RowOp> row_ops[G];
     struct Ranked { int rank; int row; int32_t hi; SweepOpHost op; };
     std::vector<std::vector<Ranked>> by_chunk;
-    std::vector<int32_t> count; // ops of (row, chunk)
     for (size_t rg = 0; rg < n_rg; rg++) {
         const size_t r_begin = rg * G, r_end = std::min(n_rows, (rg + 1) * G);
         // the chunks this row group touches, ascending
@@ -52,7 +51,6 @@ void build_sweep_plan(const int32_t *row_ptr, const int32_t *col_idx, size_t mb,
         out.rg_chunk_ptr[rg + 1] = (int32_t)out.chunk_ids.size();
 
         // ---- ops of every block row: neighbouring blocks in pairs; w3 gets the local row later ----
-        count.assign((size_t)G * std::max<size_t>(n_chunks, 1), 0);
         for (int lr = 0; lr < G; lr++) {
             row_ops[lr].clear();
             if (r_begin + (size_t)lr >= r_end) continue;
@@ -99,128 +97,142 @@ void build_sweep_plan(const int32_t *row_ptr, const int32_t *col_idx, size_t mb,
                 // While chunk p is swept, chunks p - 1, p and p + 1 are in LDS: the op may run in any period p with
                 // p - 1 <= cl0 and cl_hi <= p + 1.
                 const int32_t first = std::max(cl_hi - 1, 0), last = std::min<int32_t>(cl0 + 1, (int32_t)n_chunks - 1);
-                const int32_t exec = std::min(std::max(cl_hi, first), last);
                 (pair ? out.n_pairs : out.n_singles)++;
-                row_ops[lr].push_back(RowOp{exec, first, last, cl_hi, op});
-                count[(size_t)lr * n_chunks + (size_t)exec]++;
+                row_ops[lr].push_back(RowOp{first, last, cl_hi, op});
                 q += pair ? 2 : 1;
             }
         }
 
-        // ---- block rows -> wavefronts.  All wavefronts meet at a barrier once per chunk, so the cost of a chunk
-        // is the op count of its busiest wavefront: start from the block rows in order, then swap pairs of rows
-        // between wavefronts while the sum over chunks of that maximum falls (deterministic, a few passes). ----
+        // ---- block rows -> wavefronts, and which period every op runs in.  All wavefronts meet at a barrier once per
+        // period, so a period costs the op count of its busiest wavefront, and an op may run in any period of its
+        // window [first, last] (at most three periods).  For a given row assignment the cheapest common caps c_p
+        // (every wavefront runs at most c_p ops in period p) are found by going through the periods once: a wavefront
+        // that runs its pending ops earliest deadline first, as many as the caps allow, is left at period p with the
+        // ops that HAVE to run now, and c_p is the largest such count over the wavefronts (capacity is added as late
+        // as possible, where it serves the most windows; with unit jobs and interval windows no other caps have a
+        // smaller sum).  Pending ops of a wavefront are three counters (deadline p, p + 1, p + 2), so the sum of the
+        // caps of an assignment costs O(periods x wavefronts).  The assignment: rows in descending op count to the
+        // wavefront with the fewest ops so far, then swaps of two rows between wavefronts while the sum of the caps
+        // falls (deterministic, bounded work per row group). ----
         int wave_of[G];
         for (int lr = 0; lr < G; lr++) wave_of[lr] = lr / RW;
+        std::vector<int32_t> caps(n_chunks, MIN_OPS);
         if (n_chunks > 0) {
-            std::vector<int32_t> load((size_t)WAVES * n_chunks, 0);
-            for (int lr = 0; lr < G; lr++)
-                for (size_t c = 0; c < n_chunks; c++) load[(size_t)wave_of[lr] * n_chunks + c] += count[(size_t)lr * n_chunks + c];
-            auto chunk_cost = [&](size_t c) {
-                int32_t m = MIN_OPS;
-                for (int w = 0; w < WAVES; w++) m = std::max(m, load[(size_t)w * n_chunks + c]);
-                return m;
+            const size_t n = n_chunks;
+            {
+                int order[G], n_rows_of[WAVES] = {0};
+                long total_of[WAVES] = {0};
+                for (int lr = 0; lr < G; lr++) order[lr] = lr;
+                std::stable_sort(order, order + G, [&](int x, int y) { return row_ops[x].size() > row_ops[y].size(); });
+                for (int k = 0; k < G; k++) {
+                    int best = -1;
+                    for (int w = 0; w < WAVES; w++)
+                        if (n_rows_of[w] < RW && (best < 0 || total_of[w] < total_of[best])) best = w;
+                    wave_of[order[k]] = best;
+                    n_rows_of[best]++;
+                    total_of[best] += (long)row_ops[order[k]].size();
+                }
+            }
+            std::vector<int32_t> win((size_t)WAVES * n * 3, 0); // ops of wavefront w with window [first, first + len]: win[(w * n + first) * 3 + len]
+            auto add_row = [&](int lr, int w, int32_t sign) {
+                for (const RowOp &ro : row_ops[lr]) win[((size_t)w * n + (size_t)ro.first) * 3 + (size_t)(ro.last - ro.first)] += sign;
             };
-            for (int pass = 0; pass < 4; pass++) {
+            for (int lr = 0; lr < G; lr++) add_row(lr, wave_of[lr], 1);
+            auto sum_of_caps = [&](std::vector<int32_t> *caps_out) {
+                long sum = 0;
+                int32_t pend[WAVES][3] = {{0}};
+                for (size_t p = 0; p < n; p++) {
+                    int32_t cap = MIN_OPS;
+                    for (int w = 0; w < WAVES; w++) {
+                        const int32_t *c = &win[((size_t)w * n + p) * 3];
+                        pend[w][0] += c[0]; pend[w][1] += c[1]; pend[w][2] += c[2];
+                        cap = std::max(cap, pend[w][0]);
+                    }
+                    for (int w = 0; w < WAVES; w++) {
+                        // the ops due now run; what is left of the cap goes to the next deadlines, but the last pending op
+                        // stays for the next period when it may (see the schedule below)
+                        int32_t room = cap - pend[w][0];
+                        if (p + 1 < n && room >= pend[w][1] + pend[w][2] && pend[w][1] + pend[w][2] > 0) room = pend[w][1] + pend[w][2] - 1;
+                        const int32_t r1 = std::min(room, pend[w][1]);
+                        room -= r1;
+                        const int32_t r2 = std::min(room, pend[w][2]);
+                        pend[w][0] = pend[w][1] - r1;
+                        pend[w][1] = pend[w][2] - r2;
+                        pend[w][2] = 0;
+                    }
+                    sum += cap;
+                    if (caps_out) (*caps_out)[p] = cap;
+                }
+                return sum;
+            };
+            long best = sum_of_caps(nullptr);
+            // work bound: about 2e8 counter updates per plan, shared evenly by the row groups
+            long budget = (long)(2e8 / (double)(n * WAVES * 3) / (double)n_rg);
+            for (int pass = 0; pass < 4 && budget > 0; pass++) {
                 bool improved = false;
-                for (int i = 0; i < G; i++)
-                    for (int j = i + 1; j < G; j++) {
+                for (int i = 0; i < G && budget > 0; i++)
+                    for (int j = i + 1; j < G && budget > 0; j++) {
                         const int wi = wave_of[i], wj = wave_of[j];
-                        if (wi == wj) continue;
-                        long delta = 0;
-                        for (size_t c = 0; c < n_chunks; c++) {
-                            const int32_t d = count[(size_t)j * n_chunks + c] - count[(size_t)i * n_chunks + c];
-                            if (d == 0) continue;
-                            const int32_t before = chunk_cost(c);
-                            load[(size_t)wi * n_chunks + c] += d;
-                            load[(size_t)wj * n_chunks + c] -= d;
-                            delta += chunk_cost(c) - before;
-                            load[(size_t)wi * n_chunks + c] -= d;
-                            load[(size_t)wj * n_chunks + c] += d;
-                        }
-                        if (delta < 0) {
-                            for (size_t c = 0; c < n_chunks; c++) {
-                                const int32_t d = count[(size_t)j * n_chunks + c] - count[(size_t)i * n_chunks + c];
-                                load[(size_t)wi * n_chunks + c] += d;
-                                load[(size_t)wj * n_chunks + c] -= d;
-                            }
+                        if (wi == wj || (row_ops[i].empty() && row_ops[j].empty())) continue;
+                        add_row(i, wi, -1); add_row(i, wj, 1); add_row(j, wj, -1); add_row(j, wi, 1);
+                        const long now = sum_of_caps(nullptr);
+                        budget--;
+                        if (now < best) {
+                            best = now;
                             std::swap(wave_of[i], wave_of[j]);
                             improved = true;
+                        } else {
+                            add_row(i, wj, -1); add_row(i, wi, 1); add_row(j, wi, -1); add_row(j, wj, 1);
                         }
                     }
                 if (!improved) break;
             }
+            sum_of_caps(&caps);
         }
 
-        // ---- which period every op runs in.  All wavefronts meet at a barrier once per period, so a period costs
-        // the op count of its busiest wavefront.  An op may run one period before or after its nominal one where
-        // its chunks are resident: every period gets a common cap (what has to run now on the busiest wavefront,
-        // or an even share of what is left), and every wavefront runs its pending ops up to the cap, earliest
-        // deadline first. ----
-        struct Pending { int32_t last, first, seq, row, hi, exec; SweepOpHost op; };
+        struct Pending { int32_t last, first, seq, row, hi; SweepOpHost op; };
         std::vector<std::vector<std::vector<Ranked>>> schedule((size_t)WAVES, std::vector<std::vector<Ranked>>(n_chunks));
         if (n_chunks > 0) {
-            std::vector<Pending> todo[WAVES];
-            size_t next[WAVES] = {0}, left = 0;
             for (int w = 0; w < WAVES; w++) {
+                std::vector<Pending> todo;
                 int r = 0;
                 for (int lr = 0; lr < G; lr++) {
                     if (wave_of[lr] != w) continue;
                     if (r_begin + (size_t)lr < r_end) out.row_map[(rg * WAVES + (size_t)w) * RW + (size_t)r] = (int32_t)row_at(r_begin + (size_t)lr);
-                    for (const RowOp &ro : row_ops[lr]) todo[w].push_back(Pending{ro.last, ro.first, (int32_t)todo[w].size(), r, ro.hi, ro.exec, ro.op});
+                    for (const RowOp &ro : row_ops[lr]) todo.push_back(Pending{ro.last, ro.first, (int32_t)todo.size(), r, ro.hi, ro.op});
                     r++;
                 }
-                std::stable_sort(todo[w].begin(), todo[w].end(), [](const Pending &a, const Pending &b) { return a.first < b.first; });
-                left += todo[w].size();
-            }
-            std::vector<Pending> ready[WAVES];
-            size_t left_w[WAVES];
-            for (int w = 0; w < WAVES; w++) left_w[w] = todo[w].size();
-            for (size_t c = 0; c < n_chunks; c++) {
-                // Per wavefront: ops whose nominal period has come (deadline order: what has to run now first), then
-                // those of the next period, which may run early.  The period costs what its busiest wavefront has to
-                // run (its musts, or its own even pace over the periods that are left); every other wavefront uses
-                // that time too, with ops of the next period if it has no others, so that they are gone before
-                // they become musts.  One op of the next period always stays: the first op of a period must not be
-                // an early one.
-                size_t due[WAVES], must[WAVES], cap = MIN_OPS;
-                for (int w = 0; w < WAVES; w++) {
-                    while (next[w] < todo[w].size() && todo[w][next[w]].first <= (int32_t)c) ready[w].push_back(todo[w][next[w]++]);
-                    std::stable_sort(ready[w].begin(), ready[w].end(), [](const Pending &a, const Pending &b) {
+                std::stable_sort(todo.begin(), todo.end(), [](const Pending &a, const Pending &b) { return a.first < b.first; });
+                std::vector<Pending> ready;
+                size_t next = 0;
+                for (size_t c = 0; c < n_chunks; c++) {
+                    while (next < todo.size() && todo[next].first <= (int32_t)c) ready.push_back(todo[next++]);
+                    std::stable_sort(ready.begin(), ready.end(), [](const Pending &a, const Pending &b) {
                         if (a.last != b.last) return a.last < b.last;
                         return a.seq < b.seq;
                     });
-                    std::stable_partition(ready[w].begin(), ready[w].end(), [&](const Pending &a) { return a.exec <= (int32_t)c; });
-                    due[w] = must[w] = 0;
-                    while (due[w] < ready[w].size() && ready[w][due[w]].exec <= (int32_t)c) due[w]++;
-                    while (must[w] < due[w] && ready[w][must[w]].last <= (int32_t)c) must[w]++;
-                    const size_t pace = (left_w[w] + (n_chunks - c) - 1) / (n_chunks - c);
-                    cap = std::max(cap, std::max(must[w], std::min(due[w], pace)));
-                }
-                for (int w = 0; w < WAVES; w++) {
-                    const size_t early = ready[w].size() - due[w];
-                    size_t k = std::max(must[w], std::min(due[w], cap));
-                    size_t pull = 0;
-                    if (k < cap && early > 1) pull = std::min(early - 1, cap - k);
-                    if (pull) { // the early ops to run sit behind the due ones that wait: bring them forward
-                        std::rotate(ready[w].begin() + (long)k, ready[w].begin() + (long)due[w], ready[w].begin() + (long)(due[w] + pull));
-                        k += pull;
-                    }
+                    // Up to the cap, earliest deadline first.  The op that opens the next period has to be one that is
+                    // ready now (its LDS reads are issued before the boundary's barrier, so its chunks must be resident
+                    // already): a wavefront that could run everything it has keeps its last op for that.
+                    size_t musts = 0;
+                    while (musts < ready.size() && ready[musts].last <= (int32_t)c) musts++;
+                    size_t k = std::min(ready.size(), (size_t)caps[c]);
+                    if (k == ready.size() && k > musts && c + 1 < n_chunks) k--;
+                    k = std::max(k, musts);
                     std::vector<Ranked> &list = schedule[(size_t)w][c];
                     for (size_t x = 0; x < k; x++) {
-                        const Pending &pe = ready[w][x];
+                        const Pending &pe = ready[x];
                         // rank = how many ops of this block row the period already holds: ops of one block
                         // row (same accumulators) end up spread over the period
                         int rank = 0;
                         for (const Ranked &y : list) rank += y.row == pe.row;
                         list.push_back(Ranked{rank, pe.row, pe.hi, pe.op});
                     }
-                    ready[w].erase(ready[w].begin(), ready[w].begin() + (long)k);
-                    left_w[w] -= k;
-                    left -= k;
+                    ready.erase(ready.begin(), ready.begin() + (long)k);
+                    if (!ready.empty() && ready.front().last <= (int32_t)c) throw std::logic_error("sweep plan: an op missed its last period");
                 }
+                if (!ready.empty() || next != todo.size()) throw std::logic_error("sweep plan: ops left over by the period schedule");
             }
-            if (left) throw std::logic_error("sweep plan: ops left over by the period schedule");
         }
 
         // ---- streams: ops of chunk 0, ops of chunk 1, ..., end; the first op of a chunk carries the chunk boundary ----

@@ -276,9 +276,10 @@ def test_headline_matrix_pairs_nearly_everything():
     assert plan["pairs"] * 2 + plan["singles"] == A["nnzb"]
     # blocks paired inside a chunk or across two consecutive chunks: few stay single, few fillers
     assert plan["singles"] < 0.12 * A["nnzb"] and plan["fillers"] < 0.01 * (plan["pairs"] + plan["singles"])
-    # ops run a period early or late where their chunks are resident: the busiest wavefront of a period has
-    # hardly more ops than the average one (1.23 x without that freedom)
-    assert plan["period_max_sum"] * WAVES < 1.08 * (plan["pairs"] + plan["singles"] + plan["fillers"])
+    # ops run a period early or late where their chunks are resident, and the rows are dealt to the wavefronts for
+    # the cheapest caps: the busiest wavefront of a period has hardly more ops than the average one (1.23 x with
+    # every op in its nominal period)
+    assert plan["period_max_sum"] * WAVES < 1.045 * (plan["pairs"] + plan["singles"] + plan["fillers"])
     per_wave = np.diff(plan["op_ptr"])
     assert per_wave.min() >= 4 * 32 + 1 and per_wave.max() <= 72 * 32
 
