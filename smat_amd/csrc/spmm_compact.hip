@@ -27,17 +27,27 @@
 //    32 columns = K of one v_mfma_f32_16x16x32_f16.  The product is formed as
 //    C^T = B^T * A^T like in the other kernels:
 //      A operand   lane (m = lane % 16, g = lane / 16): one 16-byte load from acol;
-//      B operand   lane (i = lane % 16, g) loads 8 bytes = columns 4i .. 4i+3 of row col(entry)
-//                  for each of its 8 entries (16 lanes read 128 contiguous bytes); the q-th
-//                  halves of two consecutive entries are merged with one v_perm_b32 into the
-//                  operand word of n-tile q, so tile q of a 64-column group owns columns 4i + q;
-//      result      lane (m, g) holds rows i = 4g .. 4g+3 of the four tiles = 16 consecutive
-//                  columns of C row m: two 16-byte stores (fp16) per 64-column group.
+//      B operand   lane (i = lane % 16, g) needs, for each of its 8 entries (listed columns 8g .. 8g+7 of the
+//                  step), the columns of C its tiles own.  Every gather is 16 bytes per lane: a CU keeps a
+//                  limited number of vector memory instructions (and of cache lines) in flight, so an
+//                  instruction should bring as much as it can (8-byte gathers: 12 % slower on every config).
+//                  TQ even: 8 columns 8i .. 8i+7 of a 128-column group per entry (16 lanes read 256
+//                  contiguous bytes); one v_perm_b32 per word merges the t-th halves of two consecutive
+//                  entries into the operand word of n-tile t, so tile t of the group owns columns 8i + t.
+//                  TQ = 1 (rows of 128 bytes): lanes i < 8 gather the even entries of the group, lanes
+//                  i >= 8 the odd ones, 8 columns 8 (i & 7) .. + 7 each (4 instructions, not 8); lane i and
+//                  lane i ^ 8 then trade halves (one DPP row rotation per word), so that each has 4 columns
+//                  of all 8 entries: tile t owns columns 8 (i & 7) + 4 (i >> 3) + t.
+//                  The index list keeps, inside every group of 8, the even entries first and then the odd
+//                  ones, so the four indices such a lane needs are one 16-byte load.
+//      result      TQ even: lane (m, g) holds 32 consecutive columns of C row m per 128-column group;
+//                  TQ = 1: after one v_permlane32_swap per value, 16 consecutive columns.
 #include <hip/hip_runtime.h>
 #include <hipcub/hipcub.hpp>
 #include <stdint.h>
 
 #include <algorithm>
+#include <type_traits>
 #include <vector>
 
 #include "devmem.h"
@@ -124,7 +134,9 @@ __global__ void gather_kernel(const uint16_t *__restrict__ vals, const uint16_t 
     while (m) {
         const int k = __ffs(m) - 1;
         m &= m - 1;
-        cols[o] = c0 + k;
+        // inside its group of 8 the even entries come first, then the odd ones: the lanes of the product kernel that
+        // gather the even (odd) entries of a group read their four indices with one 16-byte load
+        cols[(o & ~7L) + ((o & 1) << 2) + ((o & 7) >> 1)] = c0 + k;
         uint16_t *dst = acol + ((o >> 3) * 16) * 8 + (o & 7); // (step*4 + g) = o / 8
 #pragma unroll
         for (int r = 0; r < 16; r++) dst[r * 8] = blk[r * 16 + k];
@@ -186,11 +198,8 @@ __global__ __launch_bounds__(256) void transpose_b_kernel(const uint16_t *__rest
 
 // ---- the product ----
 
-#ifndef COMPACT_KERNEL_ATTR
-#define COMPACT_KERNEL_ATTR
-#endif
 template <int TQ, bool C_F32>
-__global__ __launch_bounds__(256) COMPACT_KERNEL_ATTR void spmm_compact_kernel(
+__global__ __launch_bounds__(256) void spmm_compact_kernel(
     const uint16_t *__restrict__ acol, const int32_t *__restrict__ cols, const uint16_t *__restrict__ Bt,
     void *__restrict__ Cout, float *__restrict__ workspace, const WorkItem *__restrict__ items, int n_items, int N,
     int n_panels, long panel_stride, long row_stride)
@@ -204,13 +213,8 @@ __global__ __launch_bounds__(256) COMPACT_KERNEL_ATTR void spmm_compact_kernel(
     const long wg = (long)(blockIdx.x & 7) * chunk + (blockIdx.x >> 3);
     const long w = wg * 4 + wave;
     if (w >= total) return;
-#ifdef COMPACT_ITEM_MAJOR
-    const int it = (int)(w / n_panels);
-    const int panel = (int)(w - (long)it * n_panels);
-#else
     const int panel = (int)(w / n_items);
     const int it = (int)(w - (long)panel * n_items);
-#endif
     const WorkItem wi = items[it];
     const int br = __builtin_amdgcn_readfirstlane(wi.block_row);
     const int e0 = __builtin_amdgcn_readfirstlane(wi.begin);
@@ -222,11 +226,21 @@ __global__ __launch_bounds__(256) COMPACT_KERNEL_ATTR void spmm_compact_kernel(
     // Row `col` of this panel of B starts at Bp + col * row_stride (B in place: panel_stride = PANEL,
     // row_stride = N; the transposed copy: panels one after the other, row_stride = PANEL).
     const uint16_t *Bp = Bt + (long)panel * panel_stride;
-    int boff[TQ]; // element offset of this lane's 4 columns inside the panel row (its column 0 when out of range)
+    // Every gather is 16 bytes per lane: what a CU can keep in flight is a number of vector memory instructions
+    // and of cache lines, so an instruction should bring as much as it can.
+    //   WIDE (TQ even): a lane takes 8 columns of a 128-column group, for each of its 8 entries.
+    //   PAIRED (TQ = 1, rows of 128 bytes): lanes i16 < 8 take the even entries, lanes i16 >= 8 the odd ones, 8
+    //   columns each (4 instructions instead of 8); the two lanes then trade halves, so that each has 4 columns of
+    //   all 8 entries again.
+    constexpr bool WIDE = TQ % 2 == 0, PAIRED = TQ == 1;
+    static_assert(WIDE || PAIRED, "panel widths: 64 or a multiple of 128 columns");
+    constexpr int NG = WIDE ? TQ / 2 : 1; // groups of 128 columns (WIDE)
+    const bool odd_entries = (i16 & 8) != 0; // PAIRED
+    int boff[NG]; // element offset of this lane's 8 columns inside the panel row (its column 0 when out of range)
 #pragma unroll
-    for (int q = 0; q < TQ; q++) {
-        const int n = 64 * q + 4 * i16;
-        boff[q] = n0 + n < N ? n : 0; // N % 8 == 0: all four columns or none
+    for (int q = 0; q < NG; q++) {
+        const int n = WIDE ? 128 * q + 8 * i16 : 8 * (i16 & 7);
+        boff[q] = n0 + n < N ? n : 0; // N % 8 == 0: all of the lane's columns or none
     }
 
     f32x4 acc[TQ][4];
@@ -239,37 +253,65 @@ __global__ __launch_bounds__(256) COMPACT_KERNEL_ATTR void spmm_compact_kernel(
     // column indices of step s+2, then the operands of step s+1 (whose indices arrived a step
     // ago) are requested before the MFMAs of step s.  Loads past the end of the item read the
     // next item's data or the padding behind the arrays: always valid addresses, never used.
-    struct Entries { u32x4 r[2]; };
-    struct Operands { u32x4 aw; uint2 L[TQ][8]; };
+    struct Entries { u32x4 r[PAIRED ? 1 : 2]; }; // the indices of a group of 8: entries 0, 2, 4, 6, then 1, 3, 5, 7
+    struct Operands { u32x4 aw; u32x4 L[NG][PAIRED ? 4 : 8]; };
     auto load_entries = [&](int e, Entries &x) {
         const u32x4 *lp = reinterpret_cast<const u32x4 *>(cols + e + 8 * g);
-        x.r[0] = lp[0]; x.r[1] = lp[1];
+        if constexpr (PAIRED) {
+            x.r[0] = lp[odd_entries ? 1 : 0];
+        } else {
+            x.r[0] = lp[0]; x.r[1] = lp[1];
+        }
     };
     auto load_operands = [&](int e, const Entries &x, Operands &o) {
-        const uint32_t col[8] = {x.r[0][0], x.r[0][1], x.r[0][2], x.r[0][3], x.r[1][0], x.r[1][1], x.r[1][2], x.r[1][3]};
         o.aw = *reinterpret_cast<const u32x4 *>(acol + ((long)(e >> 3) + g) * 128 + i16 * 8);
+        if constexpr (PAIRED) {
 #pragma unroll
-        for (int q = 0; q < TQ; q++)
+            for (int j = 0; j < 4; j++)
+                o.L[0][j] = *reinterpret_cast<const u32x4 *>(Bp + (long)x.r[0][j] * row_stride + boff[0]); // entry 2j or 2j + 1
+        } else {
 #pragma unroll
-            for (int j = 0; j < 8; j++)
-                o.L[q][j] = *reinterpret_cast<const uint2 *>(Bp + (long)col[j] * row_stride + boff[q]);
+            for (int q = 0; q < NG; q++)
+#pragma unroll
+                for (int j = 0; j < 8; j++)
+                    o.L[q][j] = *reinterpret_cast<const u32x4 *>(Bp + (long)x.r[j & 1][j >> 1] * row_stride + boff[q]);
+        }
     };
     auto multiply = [&](const Operands &o) {
         const f16x8 av = __builtin_bit_cast(f16x8, o.aw);
+        if constexpr (WIDE) {
 #pragma unroll
-        for (int q = 0; q < TQ; q++) {
-            // tile t of the group takes the t-th of the four columns: words = (entry 2p, entry 2p+1)
+            for (int q = 0; q < NG; q++)
+#pragma unroll
+                for (int t = 0; t < 8; t++) { // tile t of the group takes the t-th of the lane's eight columns
+                    u32x4 b;
+#pragma unroll
+                    for (int p = 0; p < 4; p++)
+                        b[p] = __builtin_amdgcn_perm(o.L[q][2 * p + 1][t >> 1], o.L[q][2 * p][t >> 1], (t & 1) ? 0x07060302u : 0x05040100u);
+                    acc[2 * q + (t >> 2)][t & 3] = __builtin_amdgcn_mfma_f32_16x16x32_f16(__builtin_bit_cast(f16x8, b), av, acc[2 * q + (t >> 2)][t & 3], 0, 0, 0);
+                }
+        } else {
+            // Lane i16 < 8 holds columns 8 i16 .. + 7 of the even entries, lane i16 + 8 the same columns of the odd
+            // entries.  Each sends the half the other needs (row rotation by 8 lanes) and ends up with 4 columns of
+            // both entries of every pair: columns 8 (i16 & 7) + 4 (i16 >> 3) + t, t = tile.
             u32x4 b[4];
 #pragma unroll
             for (int p = 0; p < 4; p++) {
-                b[0][p] = __builtin_amdgcn_perm(o.L[q][2 * p + 1].x, o.L[q][2 * p].x, 0x05040100u);
-                b[1][p] = __builtin_amdgcn_perm(o.L[q][2 * p + 1].x, o.L[q][2 * p].x, 0x07060302u);
-                b[2][p] = __builtin_amdgcn_perm(o.L[q][2 * p + 1].y, o.L[q][2 * p].y, 0x05040100u);
-                b[3][p] = __builtin_amdgcn_perm(o.L[q][2 * p + 1].y, o.L[q][2 * p].y, 0x07060302u);
+                const u32x4 x = o.L[0][p];
+                const uint32_t s0 = odd_entries ? x[0] : x[2], s1 = odd_entries ? x[1] : x[3];
+                const uint32_t k0 = odd_entries ? x[2] : x[0], k1 = odd_entries ? x[3] : x[1];
+                const uint32_t r0 = (uint32_t)__builtin_amdgcn_update_dpp(0, (int)s0, 0x128, 0xf, 0xf, false); // row_ror:8
+                const uint32_t r1 = (uint32_t)__builtin_amdgcn_update_dpp(0, (int)s1, 0x128, 0xf, 0xf, false);
+                const uint32_t ev0 = odd_entries ? r0 : k0, ev1 = odd_entries ? r1 : k1; // entry 2p
+                const uint32_t od0 = odd_entries ? k0 : r0, od1 = odd_entries ? k1 : r1; // entry 2p + 1
+                b[0][p] = __builtin_amdgcn_perm(od0, ev0, 0x05040100u);
+                b[1][p] = __builtin_amdgcn_perm(od0, ev0, 0x07060302u);
+                b[2][p] = __builtin_amdgcn_perm(od1, ev1, 0x05040100u);
+                b[3][p] = __builtin_amdgcn_perm(od1, ev1, 0x07060302u);
             }
 #pragma unroll
             for (int t = 0; t < 4; t++)
-                acc[q][t] = __builtin_amdgcn_mfma_f32_16x16x32_f16(__builtin_bit_cast(f16x8, b[t]), av, acc[q][t], 0, 0, 0);
+                acc[0][t] = __builtin_amdgcn_mfma_f32_16x16x32_f16(__builtin_bit_cast(f16x8, b[t]), av, acc[0][t], 0, 0, 0);
         }
     };
     if (e0 < e1) {
@@ -293,16 +335,51 @@ __global__ __launch_bounds__(256) COMPACT_KERNEL_ATTR void spmm_compact_kernel(
         }
     }
 
-    // acc[q][t][r] = C[br*16 + i16][n0 + 64q + 16g + 4r + t]
     const long m = (long)br * 16 + i16;
+    if constexpr (WIDE) {
+        // tile t8 = 4 * (q & 1) + t of group q / 2: acc[q][t][r] = C[br*16 + i16][n0 + 128 (q/2) + 32g + 8r + t8]
 #pragma unroll
-    for (int q = 0; q < TQ; q++) {
-        const int c0 = n0 + 64 * q + 16 * g;
+        for (int q2 = 0; q2 < NG; q2++) {
+            const int c0 = n0 + 128 * q2 + 32 * g;
+            float o[32];
+#pragma unroll
+            for (int r = 0; r < 4; r++)
+#pragma unroll
+                for (int t = 0; t < 8; t++) o[8 * r + t] = acc[2 * q2 + (t >> 2)][t & 3][r];
+            if (dst >= 0 || C_F32) {
+                float *row = dst >= 0 ? workspace + ((long)dst * 16 + i16) * (long)N
+                                      : reinterpret_cast<float *>(Cout) + m * (long)N;
+#pragma unroll
+                for (int h = 0; h < 8; h++)
+                    if (c0 + 4 * h < N)
+                        *reinterpret_cast<f32x4 *>(row + c0 + 4 * h) = (f32x4){o[4 * h], o[4 * h + 1], o[4 * h + 2], o[4 * h + 3]};
+            } else {
+                uint16_t *row = reinterpret_cast<uint16_t *>(Cout) + m * (long)N;
+#pragma unroll
+                for (int h = 0; h < 4; h++) {
+                    f16x8 v;
+#pragma unroll
+                    for (int j = 0; j < 8; j++) v[j] = (_Float16)o[8 * h + j];
+                    if (c0 + 8 * h < N) *reinterpret_cast<f16x8 *>(row + c0 + 8 * h) = v;
+                }
+            }
+        }
+    } else {
+        // acc[0][t][r] = C[br*16 + i16][n0 + cb + t] with cb = 32 g + 8 r (g < 2) or 32 (g - 2) + 8 r + 4 (g >= 2): lane
+        // (i16, g) and lane (i16, g + 2) hold the two halves of the same 8-column groups.  One swap per value between
+        // the halves of the wavefront (the lower lanes hand over r = 2, 3 and get r = 0, 1) leaves every lane with 16
+        // consecutive columns, starting at 32 (g & 1) + 16 (g >> 1).
         float o[16];
 #pragma unroll
-        for (int r = 0; r < 4; r++)
+        for (int t = 0; t < 4; t++)
 #pragma unroll
-            for (int t = 0; t < 4; t++) o[4 * r + t] = acc[q][t][r];
+            for (int rr = 0; rr < 2; rr++) {
+                const float lo = acc[0][t][rr], hi = acc[0][t][rr + 2]; // scalars first: a bit cast of a vector element reads element 0
+                const auto sw = __builtin_amdgcn_permlane32_swap(__float_as_uint(lo), __float_as_uint(hi), false, false);
+                o[8 * rr + t] = __uint_as_float((uint32_t)sw[0]);
+                o[8 * rr + 4 + t] = __uint_as_float((uint32_t)sw[1]);
+            }
+        const int c0 = n0 + 32 * (g & 1) + 16 * (g >> 1);
         if (dst >= 0 || C_F32) {
             float *row = dst >= 0 ? workspace + ((long)dst * 16 + i16) * (long)N
                                   : reinterpret_cast<float *>(Cout) + m * (long)N;
@@ -383,11 +460,7 @@ hipError_t launch_compact(const CompactArgs &a_in, hipStream_t st)
     int tq = 1;
     if (a.N >= 256 && items * (long)(a.N / 256) >= 4096) tq = 4;
     else if (a.N >= 128 && items * (long)(a.N / 128) >= 2048) tq = 2;
-#ifdef COMPACT_FORCE_TQ
-    tq = COMPACT_FORCE_TQ;
-#else
     while (tq > 1 && a.K * (size_t)(64 * tq) * sizeof(uint16_t) > ((size_t)128 << 20)) tq >>= 1;
-#endif
     if (tq == 4) e = launch_compact_tq<4>(a, st);
     else if (tq == 2) e = launch_compact_tq<2>(a, st);
     else e = launch_compact_tq<1>(a, st);

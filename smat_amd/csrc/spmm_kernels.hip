@@ -426,12 +426,8 @@ hipError_t launch_rowwise(const SpmmArgs &a, hipStream_t st)
     hipError_t e;
     if (!a.b_packed && a.n_split_rows == 0 && a.max_item_blocks > 0 && a.max_item_blocks <= 2 * SHORT_NP && a.N >= 32 &&
         (long)a.n_items * (long)((a.N + 31) / 32) <= SHORT_MAX_WAVES) {
-#ifndef SMAT_SHORT_TN
         // 32-column panels while that still leaves the chip short of wavefronts, else 64
         const bool narrow = (long)a.n_items * (long)((a.N + 63) / 64) < 2048;
-#else
-        const bool narrow = SMAT_SHORT_TN == 2;
-#endif
         return narrow ? launch_rowwise_short<2>(a, st) : launch_rowwise_short<4>(a, st);
     }
     if (a.b_packed) {
