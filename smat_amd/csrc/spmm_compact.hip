@@ -61,6 +61,8 @@ typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
 
 namespace {
 
+int g_force_tq = 0; // test hook: 1, 2 or 4 = panels of 64, 128 or 256 columns whatever the sizes say, 0 = the launcher decides
+
 constexpr int LIST_PAD = 128; // entries readable past the end of the list (the pipeline reads up to three steps ahead)
 
 // ---- census of nonzero block columns ----
@@ -460,6 +462,7 @@ hipError_t launch_compact(const CompactArgs &a_in, hipStream_t st)
     int tq = 1;
     if (a.N >= 256 && items * (long)(a.N / 256) >= 4096) tq = 4;
     else if (a.N >= 128 && items * (long)(a.N / 128) >= 2048) tq = 2;
+    if (g_force_tq == 1 || g_force_tq == 2 || g_force_tq == 4) tq = g_force_tq;
     while (tq > 1 && a.K * (size_t)(64 * tq) * sizeof(uint16_t) > ((size_t)128 << 20)) tq >>= 1;
     if (tq == 4) e = launch_compact_tq<4>(a, st);
     else if (tq == 2) e = launch_compact_tq<2>(a, st);
@@ -624,3 +627,7 @@ hipError_t compact_build(const uint16_t *vals, const int32_t *row_ptr, const int
 }
 
 } // namespace smat
+
+// Test hook (not part of smat.h): 1, 2 or 4 = the compact kernel works on panels of 64, 128 or 256 columns whatever
+// the sizes say (each width has its own way of gathering the rows of B), 0 = the launcher decides (the default).
+extern "C" void smat_internal_compact_panel(int tq) { smat::g_force_tq = tq; }

@@ -679,6 +679,59 @@ def test_compact_kernel_config2_full_size(smat, cuda, oracle):
     assert oracle.compare(C, oracle_ref(oracle, A, B, N))[0] <= TOL_F16
 
 
+@pytest.mark.parametrize("tq", [1, 2, 4])
+def test_compact_kernel_every_panel_width(smat, cuda, oracle, tq):
+    """The compact kernel gathers the rows of B in three ways, by panel width (64, 128 or 256 columns); the launcher
+    picks the width from the sizes, so small inputs would only ever see the first.  Each is forced in turn here on the
+    same inputs: N that ends inside a panel (at any multiple of 8 columns), fp16 and fp32 results, a block row
+    long enough to be split (partial tiles through the workspace), empty rows, B row-major read in place."""
+    import ctypes as C_
+    import torch
+    lib = smat.lib
+    lib.smat_internal_compact_panel.argtypes = [C_.c_int]
+    lib.smat_internal_compact_panel.restype = None
+    lib.smat_internal_compact_panel(tq)
+    try:
+        d = gen.erdos_renyi(1024, 0.004, seed=77)               # about one nonzero per block, 1 to 3 steps per block row
+        A = bcsr_of(smat, d)
+        for N in (8, 72, 136, 264, 520):
+            B = gen.dense_b(A["K"], N, seed=N + 5, dist="normal")
+            ref = oracle_ref(oracle, A, B, N)
+            C, _ = gpu_spmm_compact(smat, cuda, A, B, N)
+            assert oracle.compare(C, ref)[0] <= TOL_F16
+            C32, _ = gpu_spmm_compact(smat, cuda, A, B, N, c_f32=True)
+            assert rel_err_f32(C32, ref) <= TOL_F32
+            assert np.array_equal(C32.astype(np.float16).view(np.uint16), C)
+        lengths = [0, 300, 1, 0, 2, 0, 0, 7] + [3] * 24         # dense blocks, one block row of 150 steps (split), empty rows
+        A = gen.random_bcsr(len(lengths), 320, 0.0, seed=6, row_lengths=lengths)
+        for N in (136, 392):
+            B = gen.dense_b(A["K"], N, seed=2 + N)
+            ref = oracle_ref(oracle, A, B, N)
+            C, _ = gpu_spmm_compact(smat, cuda, A, B, N)
+            assert oracle.compare(C, ref)[0] <= TOL_F16
+            assert not C.reshape(A["M"], N)[0:16].any()
+        # B row-major, read in place: the same bits as with the column-major B of the same values
+        d = gen.rmat(11, 8, seed=3)
+        A = bcsr_of(smat, d)
+        N, M, K, nnzb = 200, A["M"], A["K"], A["nnzb"]
+        B = gen.dense_b(K, N, seed=4, dist="uniform")
+        C_col, _ = gpu_spmm_compact(smat, cuda, A, B, N)
+        B_row = np.ascontiguousarray(B.reshape(N, K).T).reshape(-1)
+        vals, rp, ci = (to_dev(torch, A["b_val"], cuda), to_dev(torch, A["b_row_ptr"].astype(np.int32), cuda),
+                        to_dev(torch, A["b_col_idx"].astype(np.int32), cuda))
+        Bd = to_dev(torch, B_row, cuda)
+        Cd = torch.full((M, N), 0x7E00, dtype=torch.int16, device=cuda)
+        p = smat.Plan(A["b_row_ptr"], M, K, nnzb, N, col_idx_host=A["b_col_idx"], kernel=COMPACT)
+        p.attach_values(vals, rp, ci)
+        smat.spmm(vals, rp, ci, Bd, Cd, M, N, K, nnzb, plan=p, kernel=COMPACT, b_row_major=True)
+        torch.cuda.synchronize()
+        p.close()
+        assert np.array_equal(Cd.cpu().numpy().view(np.uint16), C_col)
+        assert oracle.compare(C_col, oracle_ref(oracle, A, B, N))[0] <= TOL_F16
+    finally:
+        lib.smat_internal_compact_panel(0)
+
+
 def test_compact_kernel_power_law_rows(smat, cuda, oracle):
     """R-MAT scale 15: block rows of very different length, the longest split into chunks."""
     d = gen.rmat(15, 16, seed=21)
