@@ -31,7 +31,7 @@
 //                  step), the columns of C its tiles own.  Every gather is 16 bytes per lane: a CU keeps a
 //                  limited number of vector memory instructions (and of cache lines) in flight, so an
 //                  instruction should bring as much as it can (8-byte gathers: 12 % slower on every config).
-//                  TQ even: 8 columns 8i .. 8i+7 of a 128-column group per entry (16 lanes read 256
+//                  TQ = 2: 8 columns 8i .. 8i+7 of the 128-column panel per entry (16 lanes read 256
 //                  contiguous bytes); one v_perm_b32 per word merges the t-th halves of two consecutive
 //                  entries into the operand word of n-tile t, so tile t of the group owns columns 8i + t.
 //                  TQ = 1 (rows of 128 bytes): lanes i < 8 gather the even entries of the group, lanes
@@ -40,7 +40,7 @@
 //                  of all 8 entries: tile t owns columns 8 (i & 7) + 4 (i >> 3) + t.
 //                  The index list keeps, inside every group of 8, the even entries first and then the odd
 //                  ones, so the four indices such a lane needs are one 16-byte load.
-//      result      TQ even: lane (m, g) holds 32 consecutive columns of C row m per 128-column group;
+//      result      TQ = 2: lane (m, g) holds 32 consecutive columns of C row m;
 //                  TQ = 1: after one v_permlane32_swap per value, 16 consecutive columns.
 #include <hip/hip_runtime.h>
 #include <hipcub/hipcub.hpp>
@@ -61,7 +61,7 @@ typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
 
 namespace {
 
-int g_force_tq = 0; // test hook: 1, 2 or 4 = panels of 64, 128 or 256 columns whatever the sizes say, 0 = the launcher decides
+int g_force_tq = 0; // test hook: 1 or 2 = panels of 64 or 128 columns whatever the sizes say, 0 = the launcher decides
 
 constexpr int LIST_PAD = 128; // entries readable past the end of the list (the pipeline reads up to three steps ahead)
 
@@ -230,12 +230,12 @@ __global__ __launch_bounds__(256) void spmm_compact_kernel(
     const uint16_t *Bp = Bt + (long)panel * panel_stride;
     // Every gather is 16 bytes per lane: what a CU can keep in flight is a number of vector memory instructions
     // and of cache lines, so an instruction should bring as much as it can.
-    //   WIDE (TQ even): a lane takes 8 columns of a 128-column group, for each of its 8 entries.
+    //   WIDE (TQ = 2): a lane takes 8 columns of the 128-column panel, for each of its 8 entries.
     //   PAIRED (TQ = 1, rows of 128 bytes): lanes i16 < 8 take the even entries, lanes i16 >= 8 the odd ones, 8
     //   columns each (4 instructions instead of 8); the two lanes then trade halves, so that each has 4 columns of
     //   all 8 entries again.
     constexpr bool WIDE = TQ % 2 == 0, PAIRED = TQ == 1;
-    static_assert(WIDE || PAIRED, "panel widths: 64 or a multiple of 128 columns");
+    static_assert(TQ == 1 || TQ == 2, "panels of 64 or 128 columns");
     constexpr int NG = WIDE ? TQ / 2 : 1; // groups of 128 columns (WIDE)
     const bool odd_entries = (i16 & 8) != 0; // PAIRED
     int boff[NG]; // element offset of this lane's 8 columns inside the panel row (its column 0 when out of range)
@@ -453,19 +453,19 @@ hipError_t launch_compact(const CompactArgs &a_in, hipStream_t st)
     CompactArgs a = a_in;
     hipError_t e = hipSuccess;
     if (a.b_row_major) a.Bt = const_cast<uint16_t *>(a.B); // read in place, never written
-    // Wide panels reuse the A operand over more columns; narrow ones give more wavefronts.  The
-    // panels are swept one after the other, so the rows of B that the gathers hit at random come
-    // from one panel at a time: a panel is kept under half of the 256 MiB memory-side cache (the
-    // lists of A and the rows of C stream through it too).  On a 2^20-row B at N = 128 the panel
-    // of 64 columns (128 MiB) takes 0.74 x the time of the panel of 128.
+    // Panels of 128 columns read the A operand and the indices half as often as panels of 64; those of 64 give twice
+    // the wavefronts.  Measured (N = 256 .. 4096): 128 wins where the items are long (dense blocks, 25 steps per
+    // block row: 218 against 244 us), 64 where they are short (one nonzero per block, 4 to 8 steps: 21.7 against
+    // 22.5 us, 94 against 97 us); panels of 256 columns never won.  The panels are swept one after the other, so the
+    // rows of B that the gathers hit at random come from one panel at a time: a panel is kept under half of the
+    // 256 MiB memory-side cache (the lists of A and the rows of C stream through it too).  On a 2^20-row B at
+    // N = 128 the panel of 64 columns (128 MiB) takes 0.74 x the time of the panel of 128.
     const long items = a.plan->n_items;
     int tq = 1;
-    if (a.N >= 256 && items * (long)(a.N / 256) >= 4096) tq = 4;
-    else if (a.N >= 128 && items * (long)(a.N / 128) >= 2048) tq = 2;
-    if (g_force_tq == 1 || g_force_tq == 2 || g_force_tq == 4) tq = g_force_tq;
+    if (a.N >= 128 && items * (long)(a.N / 128) >= 2048 && a.plan->n_cols >= (int64_t)items * 384) tq = 2;
+    if (g_force_tq == 1 || g_force_tq == 2) tq = g_force_tq;
     while (tq > 1 && a.K * (size_t)(64 * tq) * sizeof(uint16_t) > ((size_t)128 << 20)) tq >>= 1;
-    if (tq == 4) e = launch_compact_tq<4>(a, st);
-    else if (tq == 2) e = launch_compact_tq<2>(a, st);
+    if (tq == 2) e = launch_compact_tq<2>(a, st);
     else e = launch_compact_tq<1>(a, st);
     if (e != hipSuccess) return e;
     if (a.plan->n_split_rows > 0)
@@ -628,6 +628,6 @@ hipError_t compact_build(const uint16_t *vals, const int32_t *row_ptr, const int
 
 } // namespace smat
 
-// Test hook (not part of smat.h): 1, 2 or 4 = the compact kernel works on panels of 64, 128 or 256 columns whatever
-// the sizes say (each width has its own way of gathering the rows of B), 0 = the launcher decides (the default).
+// Test hook (not part of smat.h): 1 or 2 = the compact kernel works on panels of 64 or 128 columns whatever the sizes
+// say (each width has its own way of gathering the rows of B), 0 = the launcher decides (the default).
 extern "C" void smat_internal_compact_panel(int tq) { smat::g_force_tq = tq; }
