@@ -530,12 +530,12 @@ static int smat_plan_attach_values_impl(smat_plan *p, const uint16_t *vals, cons
     bool dense_packed = p->d_bpack != nullptr; // row-wise route: B repacked slab-major first?
     if (mixed && !dense_sweep_possible && want != SMAT_KERNEL_MIXED) {
         // Row-wise route for the dense rows: it has to beat the compact kernel on those very rows, launch and (when B
-        // is repacked for it) the extra pass over B included.  Rates as measured: the compact kernel and the row-wise
-        // kernel on B in place gather about 8 TB/s of operand bytes, the row-wise kernel on repacked B 20 TB/s; a
+        // is repacked for it) the extra pass over B included.  Rates as measured: the compact kernel gathers about 10 TB/s of
+        // operand bytes, the row-wise kernel on B in place 7.6 TB/s, the row-wise kernel on repacked B 20 TB/s; a
         // pass over B moves 4*K*N bytes at 4 TB/s; a launch costs 3 us.  (27-point stencil on 64^3 after the reorder,
-        // N = 64: a sixth of the blocks sit in dense rows, 13 us of compact kernel against 20 us for the repack alone.)
+        // N = 64: a sixth of the blocks sit in dense rows, 10 us of compact kernel against 20 us for the repack alone.)
         const double dense_cols = (double)(c->n_cols_all - c->n_cols);
-        const double t_compact = dense_cols * (double)p->n_cap * 2.0 / 8e6;
+        const double t_compact = dense_cols * (double)p->n_cap * 2.0 / 10e6;
         const double gather = (double)blocks_dense * 16.0 * (double)p->n_cap * 2.0;
         const double t_direct = gather / 7.6e6 + 3.0;
         const double t_packed = gather / 20e6 + 6.0 + 4.0 * (double)p->K * (double)p->n_cap / 4e6;
