@@ -320,9 +320,23 @@ __global__ __launch_bounds__(256) void spmm_reduce_kernel(const float *__restric
     const int i = (int)(rem / quads);
     const int q = (int)(rem - (long)i * quads);
     const SplitRow sr = rows[r];
-    f32x4 s = {0.f, 0.f, 0.f, 0.f};
-    for (int slot = sr.slot_begin; slot < sr.slot_end; slot++)
-        s += *reinterpret_cast<const f32x4 *>(workspace + ((long)slot * 16 + i) * (long)N + 4 * q);
+    // Four running sums, slot k into sum k % 4 (a fixed order: the result does not depend on the launch): the loads of
+    // four slots are under way at a time instead of one, which is what a block row of many slots waits for.
+    const float *base = workspace + (long)i * (long)N + 4 * q;
+    const long slot_stride = 16L * (long)N;
+    f32x4 s0 = {0.f, 0.f, 0.f, 0.f}, s1 = s0, s2 = s0, s3 = s0;
+    int slot = sr.slot_begin;
+    for (; slot + 4 <= sr.slot_end; slot += 4) {
+        const f32x4 v0 = *reinterpret_cast<const f32x4 *>(base + (long)slot * slot_stride);
+        const f32x4 v1 = *reinterpret_cast<const f32x4 *>(base + (long)(slot + 1) * slot_stride);
+        const f32x4 v2 = *reinterpret_cast<const f32x4 *>(base + (long)(slot + 2) * slot_stride);
+        const f32x4 v3 = *reinterpret_cast<const f32x4 *>(base + (long)(slot + 3) * slot_stride);
+        s0 += v0; s1 += v1; s2 += v2; s3 += v3;
+    }
+    if (slot < sr.slot_end) s0 += *reinterpret_cast<const f32x4 *>(base + (long)slot * slot_stride);
+    if (slot + 1 < sr.slot_end) s1 += *reinterpret_cast<const f32x4 *>(base + (long)(slot + 1) * slot_stride);
+    if (slot + 2 < sr.slot_end) s2 += *reinterpret_cast<const f32x4 *>(base + (long)(slot + 2) * slot_stride);
+    const f32x4 s = (s0 + s1) + (s2 + s3);
     const long m = (long)sr.block_row * 16 + i;
     if (C_F32) {
         *reinterpret_cast<f32x4 *>(reinterpret_cast<float *>(Cout) + m * (long)N + 4 * q) = s;
