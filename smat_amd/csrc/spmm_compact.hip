@@ -39,7 +39,8 @@
 //                  lane i ^ 8 then trade halves (one DPP row rotation per word), so that each has 4 columns
 //                  of all 8 entries: tile t owns columns 8 (i & 7) + 4 (i >> 3) + t.
 //                  The index list keeps, inside every group of 8, the even entries first and then the odd
-//                  ones, so the four indices such a lane needs are one 16-byte load.
+//                  ones, so the four indices such a lane needs are 16 contiguous bytes; one load instruction
+//                  fetches them for 8 steps at a time (lane i16 & 7 = step) and DPP row broadcasts hand them round.
 //      result      TQ = 2: lane (m, g) holds 32 consecutive columns of C row m;
 //                  TQ = 1: after one v_permlane32_swap per value, 16 consecutive columns.
 #include <hip/hip_runtime.h>
@@ -63,7 +64,7 @@ namespace {
 
 int g_force_tq = 0; // test hook: 1 or 2 = panels of 64 or 128 columns whatever the sizes say, 0 = the launcher decides
 
-constexpr int LIST_PAD = 128; // entries readable past the end of the list (the pipeline reads up to three steps ahead)
+constexpr int LIST_PAD = 640; // entries readable past the end of the list (the index loads of the 64-column panel run up to 16 steps ahead)
 
 // ---- census of nonzero block columns ----
 
@@ -258,12 +259,9 @@ __global__ __launch_bounds__(256) void spmm_compact_kernel(
     struct Entries { u32x4 r[PAIRED ? 1 : 2]; }; // the indices of a group of 8: entries 0, 2, 4, 6, then 1, 3, 5, 7
     struct Operands { u32x4 aw; u32x4 L[NG][PAIRED ? 4 : 8]; };
     auto load_entries = [&](int e, Entries &x) {
-        const u32x4 *lp = reinterpret_cast<const u32x4 *>(cols + e + 8 * g);
-        if constexpr (PAIRED) {
-            x.r[0] = lp[odd_entries ? 1 : 0];
-        } else {
-            x.r[0] = lp[0]; x.r[1] = lp[1];
-        }
+        const u32x4 *lp = reinterpret_cast<const u32x4 *>(cols + e + 8 * g); // the 128-column panel; the other has its own loop
+        x.r[0] = lp[0];
+        if constexpr (!PAIRED) x.r[1] = lp[1];
     };
     auto load_operands = [&](int e, const Entries &x, Operands &o) {
         o.aw = *reinterpret_cast<const u32x4 *>(acol + ((long)(e >> 3) + g) * 128 + i16 * 8);
@@ -316,7 +314,55 @@ __global__ __launch_bounds__(256) void spmm_compact_kernel(
                 acc[0][t] = __builtin_amdgcn_mfma_f32_16x16x32_f16(__builtin_bit_cast(f16x8, b[t]), av, acc[0][t], 0, 0, 0);
         }
     };
-    if (e0 < e1) {
+    if constexpr (PAIRED) {
+        // The index loads of 8 steps in one instruction (an instruction that brings 128 bytes costs the vector memory
+        // path as much as one that brings 1 KiB): lane (i16, g) asks for the four indices that its kind of lane (group g,
+        // even or odd entries) needs at step i16 & 7 of a block of 8 steps; at step k of the block every lane takes them
+        // from the lane that holds step k, with one DPP row broadcast per half of the 16-lane row and word.  Blocks are
+        // asked for one block ahead; what lies past the end of the item is the next item's list or the padding.
+        if (e0 < e1) {
+            auto load_block = [&](int e, u32x4 &x) {
+                x = *reinterpret_cast<const u32x4 *>(cols + e + 32 * (i16 & 7) + 8 * g + (odd_entries ? 4 : 0));
+            };
+            auto indices = [&](const u32x4 &x, auto kc, Entries &out) {
+                constexpr int K = decltype(kc)::value;
+#pragma unroll
+                for (int w = 0; w < 4; w++) {
+                    int r = __builtin_amdgcn_update_dpp(0, (int)x[w], 0x150 + K, 0xf, 0x3, false); // row_newbcast:K     -> lanes 0-7 of the row
+                    r = __builtin_amdgcn_update_dpp(r, (int)x[w], 0x150 + 8 + K, 0xf, 0xc, false); // row_newbcast:8 + K -> lanes 8-15
+                    out.r[0][w] = (uint32_t)r;
+                }
+            };
+            u32x4 blk_a, blk_b;
+            Entries ent;
+            Operands op_a, op_b;
+            load_block(e0, blk_a);
+            load_block(e0 + 256, blk_b);
+            indices(blk_a, std::integral_constant<int, 0>{}, ent);
+            load_operands(e0, ent, op_a);
+            int e = e0;
+            while (true) {
+#define SMAT_TWO_STEPS(KA, KB, BLK_B)                                                                  \
+                indices(blk_a, std::integral_constant<int, KA>{}, ent);                                \
+                load_operands(e + 32, ent, op_b);                                                      \
+                multiply(op_a);                                                                        \
+                e += 32;                                                                               \
+                if (e >= e1) break;                                                                    \
+                indices(BLK_B, std::integral_constant<int, KB>{}, ent);                                \
+                load_operands(e + 32, ent, op_a);                                                      \
+                multiply(op_b);                                                                        \
+                e += 32;                                                                               \
+                if (e >= e1) break;
+                SMAT_TWO_STEPS(1, 2, blk_a)
+                SMAT_TWO_STEPS(3, 4, blk_a)
+                SMAT_TWO_STEPS(5, 6, blk_a)
+                SMAT_TWO_STEPS(7, 0, blk_b)
+#undef SMAT_TWO_STEPS
+                blk_a = blk_b;
+                load_block(e + 256, blk_b);
+            }
+        }
+    } else if (e0 < e1) {
         Entries ent_a, ent_b;
         Operands op_a, op_b;
         load_entries(e0, ent_a);
