@@ -732,6 +732,28 @@ def test_compact_kernel_every_panel_width(smat, cuda, oracle, tq):
         lib.smat_internal_compact_panel(0)
 
 
+def test_compact_kernel_every_item_length_up_to_twenty_steps(smat, cuda, oracle):
+    """Block row r has 2 (r + 1) dense blocks = r + 1 steps of 32 columns: every item length from 1 to 20 steps, so
+    that an item ends at every position of the kernel's blocks of 8 steps (7, 8, 9, 15, 16, 17 ...), on both panel
+    widths and with rows of B that the index loads past the end of an item still have to find valid."""
+    import ctypes as C_
+    lengths = [2 * (r + 1) for r in range(20)]
+    A = gen.random_bcsr(len(lengths), 48, 0.0, seed=14, row_lengths=lengths)
+    lib = smat.lib
+    lib.smat_internal_compact_panel.argtypes = [C_.c_int]
+    lib.smat_internal_compact_panel.restype = None
+    try:
+        for tq in (1, 2):
+            lib.smat_internal_compact_panel(tq)
+            for N in (64, 200):
+                B = gen.dense_b(A["K"], N, seed=N + tq, dist="normal")
+                C32, info = gpu_spmm_compact(smat, cuda, A, B, N, c_f32=True)
+                assert info["compact_cols"] == 16 * A["nnzb"]
+                assert rel_err_f32(C32, oracle_ref(oracle, A, B, N)) <= TOL_F32
+    finally:
+        lib.smat_internal_compact_panel(0)
+
+
 def test_compact_kernel_power_law_rows(smat, cuda, oracle):
     """R-MAT scale 15: block rows of very different length, the longest split into chunks."""
     d = gen.rmat(15, 16, seed=21)
