@@ -127,6 +127,10 @@ def build_workload(name, want_b=True):
         # two kinds of block rows in one matrix (dense blocks above, about one nonzero per block below): mixed dispatch
         A = gen.half_pruned_half_er(8192, 0.10, 0.001)
         N, bdist, bseed = 4096, "normal", 0xB0000006
+    elif name == "pruned_plus_er_8192_N4096":
+        # both kinds of blocks in every block row (dense blocks, about one nonzero per block between them): mixed dispatch per block
+        A = gen.pruned_plus_er(8192, 0.10, 0.001)
+        N, bdist, bseed = 4096, "normal", 0xB0000007
     elif name == "band_4096_bw64_N128":
         d = gen.band(4096, 64)
         b = smat_amd.csr_to_bcsr(d["M"], d["K"], d["row_ptr"], d["col_idx"], d["val"])

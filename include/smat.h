@@ -101,9 +101,14 @@ int smat_plan_cache_clear(void);
 #define SMAT_KERNEL_COMPACT 5  /* only the nonzero columns of the blocks are multiplied (needs
                                * smat_plan_attach_values); for blocks with few nonzero columns */
 #define SMAT_KERNEL_MIXED 6    /* mixed dispatch inside one SpMM: block rows whose blocks are mostly full (at least
-                               * 60% of their columns nonzero) go through the row-wise kernel, the others through
-                               * the compact kernel.  Needs smat_plan_attach_values, which makes the split;
-                               * SMAT_KERNEL_AUTO takes it when each kind holds at least a tenth of the blocks */
+                               * 60% of their columns nonzero) go through a dense kernel (sweep or row-wise), the
+                               * others through the compact kernel.  Where the block rows do not sort into two kinds
+                               * but the blocks do (the classification of matrix.h:400-419), the split is per block:
+                               * the plan's copy of the mostly full blocks goes through the sweep kernel and the
+                               * compact kernel adds the columns of the other blocks to C.  Needs
+                               * smat_plan_attach_values, which makes the split; SMAT_KERNEL_AUTO takes it when each
+                               * kind holds at least a tenth of the blocks (and, per block, when its estimate of the
+                               * run time beats the better single kernel) */
 #define SMAT_KERNEL_ROWWISE_PACKED 4 /* row-wise, B always repacked (needs a plan created with this id) */
 
 typedef struct smat_spmm_opts {
@@ -166,8 +171,8 @@ int smat_plan_check(const smat_plan *plan, const int32_t *row_ptr_host, const in
 /* Fills info[0..11]: kernel id, row-wise work items, split block rows, chunk size,
  * workspace bytes, panel width, sweep stream entries, sweep (row group, K chunk) records,
  * bytes of the scratch copies of B (0 = B is read in place), nonzero block columns listed by
- * smat_plan_attach_values (0 = not attached), and for mixed dispatch the row-wise work items and the
- * blocks of the block rows that the row-wise kernel takes. */
+ * smat_plan_attach_values (0 = not attached), and for mixed dispatch the row-wise work items (-1: the
+ * split is per block, not per block row) and the blocks that the dense kernel takes. */
 int smat_plan_info(const smat_plan *plan, int64_t *info);
 
 /* Same operands as smat_spmm_bcsr_f16; C is uint16_t* or float* per opts->c_dtype.

@@ -54,6 +54,11 @@ struct smat_plan {
     };
     SweepDev sweep;       // all block rows (SMAT_KERNEL_SWEEP)
     SweepDev sweep_dense; // mixed dispatch: the block rows with mostly full blocks, when they fill the device
+    // mixed dispatch per block (rows that hold both kinds of blocks): the blocks with mostly nonzero columns, copied one
+    // behind the other into d_vals_dense, go through the sweep kernel; the compact kernel adds the other blocks' columns
+    SweepDev sweep_blocks;
+    uint16_t *d_vals_dense = nullptr;
+    int64_t n_blocks_split = 0;
     std::vector<int32_t> row_ptr_host; // the block row pointer the plan was made from: smat_plan_attach_values works from this copy
     std::vector<int32_t> col_idx_host; // kept for the split of a mixed plan (plans made with col_idx_host for AUTO / MIXED)
     uint64_t fingerprint = 0; // FNV-1a over row_ptr_host and, when given, col_idx_host
@@ -190,7 +195,7 @@ extern "C" int smat_spmm_bcsr_f16_ex(const uint16_t *vals, const int32_t *row_pt
     if (kernel == SMAT_KERNEL_SWEEP && o.kernel == SMAT_KERNEL_AUTO && !sweep_fills_device(M / 16, N))
         kernel = SMAT_KERNEL_ROWWISE;
     const uint16_t *B_as_given = B;
-    if (kernel == SMAT_KERNEL_MIXED && (!plan || !plan->compact || (!plan->d_items_dense && !plan->sweep_dense.d_ops) || !plan->d_bt || N > plan->n_cap))
+    if (kernel == SMAT_KERNEL_MIXED && (!plan || !plan->compact || (!plan->d_items_dense && !plan->sweep_dense.d_ops && !plan->sweep_blocks.d_ops) || !plan->d_bt || N > plan->n_cap))
         return set_error(SMAT_ERR_INVALID, "SMAT_KERNEL_MIXED needs a plan that split the block rows when the values were "
                                            "attached (smat_plan_attach_values) and n_hint >= N");
     if (o.b_layout == SMAT_B_ROW_MAJOR && kernel != SMAT_KERNEL_COMPACT) {
@@ -207,7 +212,14 @@ extern "C" int smat_spmm_bcsr_f16_ex(const uint16_t *vals, const int32_t *row_pt
     if (kernel == SMAT_KERNEL_MIXED) {
         // the block rows with mostly full blocks through the row-wise kernel, the others (and the empty ones) through
         // the compact kernel: disjoint rows of C, one after the other on the stream
-        if (plan->sweep_dense.d_ops) {
+        if (plan->sweep_blocks.d_ops) {
+            // per-block split: the plan's copy of the mostly full blocks through the sweep kernel (every row of C is
+            // written), then the compact kernel adds the columns of the other blocks
+            SweepArgs w{};
+            w.vals = plan->d_vals_dense; w.B = B; w.C = C; w.M = M; w.N = N; w.K = K; w.nnzb = (size_t)plan->n_blocks_split; w.c_f32 = a.c_f32;
+            plan->sweep_blocks.fill(w);
+            e = launch_sweep(w, static_cast<hipStream_t>(o.stream));
+        } else if (plan->sweep_dense.d_ops) {
             SweepArgs w{};
             w.vals = vals; w.B = B; w.C = C; w.M = M; w.N = N; w.K = K; w.nnzb = nnzb; w.c_f32 = a.c_f32;
             plan->sweep_dense.fill(w);
@@ -225,6 +237,7 @@ extern "C" int smat_spmm_bcsr_f16_ex(const uint16_t *vals, const int32_t *row_pt
             c.B = B_as_given; c.Bt = plan->d_bt; c.b_row_major = o.b_layout == SMAT_B_ROW_MAJOR; c.C = C; c.M = M; c.N = N; c.K = K;
             c.c_f32 = a.c_f32;
             c.plan = plan->compact;
+            c.accumulate = plan->sweep_blocks.d_ops != nullptr;
             e = launch_compact(c, static_cast<hipStream_t>(o.stream));
         }
     } else if (kernel == SMAT_KERNEL_COMPACT) {
@@ -494,6 +507,9 @@ static int smat_plan_attach_values_impl(smat_plan *p, const uint16_t *vals, cons
     const int dense_kernel = p->sweep.d_ops ? SMAT_KERNEL_SWEEP : SMAT_KERNEL_ROWWISE;
     auto drop_mixed = [&] {
         p->sweep_dense.release();
+        p->sweep_blocks.release();
+        if (p->d_vals_dense) { (void)dev_free(p->d_vals_dense); p->d_vals_dense = nullptr; }
+        p->n_blocks_split = 0;
         if (p->d_items_dense) { (void)dev_free(p->d_items_dense); p->d_items_dense = nullptr; }
         if (p->d_split_dense) { (void)dev_free(p->d_split_dense); p->d_split_dense = nullptr; }
         if (p->d_workspace_dense) { (void)dev_free(p->d_workspace_dense); p->d_workspace_dense = nullptr; }
@@ -511,10 +527,10 @@ static int smat_plan_attach_values_impl(smat_plan *p, const uint16_t *vals, cons
     // per block (27-point stencil) 53 us compact against 86 us row-wise; 16 per block (dense blocks, N = 4096)
     // 326 us against 180 us.  This is the per-block classification of the reference (matrix.h:400-419: blocks
     // without / with 2:4 / with dense rows) put to use per block row.
-    std::vector<uint8_t> dense;
+    std::vector<uint8_t> dense, block_cols;
     CompactPlan *c = nullptr;
     hipError_t e = compact_build(vals, row_ptr, col_idx, row_ptr_host, mb, p->nnzb, p->n_cap, may_mix ? 0.6 : 0.0,
-                                 may_mix ? &dense : nullptr, &c);
+                                 may_mix ? &dense : nullptr, &c, nullptr, may_mix ? &block_cols : nullptr);
     if (e != hipSuccess) return fail(e);
     int64_t blocks_dense = 0;
     for (size_t i = 0; may_mix && i < mb; i++)
@@ -542,8 +558,56 @@ static int smat_plan_attach_values_impl(smat_plan *p, const uint16_t *vals, cons
         dense_packed = t_packed < t_direct;
         if (std::min(t_direct, t_packed) >= 0.8 * t_compact) mixed = false;
     }
-    if (want == SMAT_KERNEL_MIXED) mixed = true;
-    if (may_mix && !mixed && blocks_dense > 0) { // the list left dense rows out: make it whole again
+    // Per-block split, where the rows do not sort into two kinds but the blocks do (the reference's classification,
+    // matrix.h:400-419, taken at its word): blocks with at least 10 of their 16 columns nonzero are copied one behind
+    // the other and go through the sweep kernel, which writes every row of C; the compact kernel then ADDS the
+    // columns of the other blocks (fp16 C: one more rounding of the partial result, well inside the tolerance).
+    // Taken when both kinds hold a tenth of the blocks, the sweep kernel's workgroups fill the device, and an
+    // estimate says it beats the better single kernel by 5 % - or when it is asked for (SMAT_KERNEL_MIXED) and the
+    // rows do not split.  Rates as measured on 8192^2, N = 4096: the sweep kernel moves its panels of B into LDS once
+    // per group of 64 block rows at 13.4 TB/s and multiplies at 1.04 Pflop/s on top of that (26,214 blocks 93 us, 79,540
+    // blocks 201 us), the compact kernel gathers 10 TB/s of rows of B, a pass over B moves 4 K N bytes at 4 TB/s + 3 us
+    // (10 % dense blocks with as many blocks again of one nonzero: estimate 179 us, measured 180; sweep kernel alone
+    // 201 us, compact kernel alone 252 us).
+    bool block_split = false;
+    std::vector<uint8_t> skip;
+    int64_t n_split_blocks = 0;
+    const double n_est = (double)p->n_cap, n_rg_est = (double)((mb + SWEEP_G - 1) / SWEEP_G);
+    auto t_sweep = [&](double blocks) { return n_rg_est * (double)p->K * n_est * 2.0 / 13.4e6 + blocks * n_est * 512.0 / 1.04e9; };
+    auto t_compact = [&](double cols) { return cols * n_est * 2.0 / 10e6; };
+    const double t_pass = 3.0 + (double)p->K * n_est / 1e6;
+    // one kernel for everything: the sweep kernel (when the plan has its work list) or the compact kernel
+    const double t_sweep_all = p->sweep.d_ops ? t_sweep((double)p->nnzb) : 1e30;
+    const double t_compact_all = t_compact((double)c->n_cols_all) + t_pass;
+    if (may_mix && !mixed && !p->col_idx_host.empty() && block_cols.size() == p->nnzb && p->nnzb < ((size_t)1 << 23) &&
+        p->K < ((size_t)1 << 28) && sweep_fills_device(mb, p->n_cap)) {
+        int64_t cols_rest = 0;
+        skip.assign(p->nnzb, 0);
+        for (size_t q = 0; q < p->nnzb; q++) {
+            if (block_cols[q] >= 10) { skip[q] = 1; n_split_blocks++; }
+            else cols_rest += block_cols[q];
+        }
+        const int64_t n_rest = (int64_t)p->nnzb - n_split_blocks;
+        if (n_split_blocks >= 2 && n_split_blocks * 10 >= (int64_t)p->nnzb && n_rest * 10 >= (int64_t)p->nnzb) {
+            const double t_split = t_sweep((double)n_split_blocks) + t_compact((double)cols_rest) + t_pass;
+            block_split = want == SMAT_KERNEL_MIXED || t_split < 0.95 * std::min(t_sweep_all, t_compact_all);
+        }
+    }
+    if (block_split) { // the list without the blocks that the sweep kernel takes
+        compact_destroy(c);
+        c = nullptr;
+        e = compact_build(vals, row_ptr, col_idx, row_ptr_host, mb, p->nnzb, p->n_cap, 0.0, nullptr, &c, skip.data(), nullptr);
+        if (e != hipSuccess) return fail(e);
+        if (c->n_split_rows > 0) { // partial tiles through the workspace cannot be added to C: one kernel for everything
+            block_split = false;
+            compact_destroy(c);
+            c = nullptr;
+            e = compact_build(vals, row_ptr, col_idx, row_ptr_host, mb, p->nnzb, p->n_cap, 0.0, nullptr, &c);
+            if (e != hipSuccess) return fail(e);
+        }
+    }
+    if (want == SMAT_KERNEL_MIXED && !block_split) mixed = true;
+    if (may_mix && !mixed && !block_split && blocks_dense > 0) { // the list left dense rows out: make it whole again
         compact_destroy(c);
         c = nullptr;
         e = compact_build(vals, row_ptr, col_idx, row_ptr_host, mb, p->nnzb, p->n_cap, 0.0, nullptr, &c);
@@ -551,8 +615,11 @@ static int smat_plan_attach_values_impl(smat_plan *p, const uint16_t *vals, cons
     }
     if (p->compact) { compact_destroy(p->compact); p->compact = nullptr; }
     drop_mixed();
-    const bool take = mixed || want == SMAT_KERNEL_COMPACT ||
-                      (want == SMAT_KERNEL_AUTO && (double)c->n_cols_all < 0.6 * 16.0 * (double)p->nnzb);
+    // the compact kernel for everything: few nonzero columns per block - unless the plan has the sweep kernel's work
+    // list and the same estimate says that one is faster (blocks of both kinds in a matrix that is dense enough)
+    const bool take = mixed || block_split || want == SMAT_KERNEL_COMPACT ||
+                      (want == SMAT_KERNEL_AUTO && (double)c->n_cols_all < 0.6 * 16.0 * (double)p->nnzb &&
+                       !(dense_kernel == SMAT_KERNEL_SWEEP && t_sweep_all < t_compact_all));
     if (!take) { // nothing will use the list: the plan keeps (or goes back to) a dense kernel
         compact_destroy(c);
         if (p->kernel == SMAT_KERNEL_COMPACT || p->kernel == SMAT_KERNEL_MIXED) p->kernel = dense_kernel;
@@ -567,7 +634,26 @@ static int smat_plan_attach_values_impl(smat_plan *p, const uint16_t *vals, cons
         if (dense_packed && !p->d_bpack && e == hipSuccess) e = dev_malloc(&p->d_bpack, p->K * p->n_cap * sizeof(uint16_t));
         if (!dense_packed && p->d_bpack && want == SMAT_KERNEL_AUTO) { (void)dev_free(p->d_bpack); p->d_bpack = nullptr; }
     }
-    if (e == hipSuccess && dense_sweep) {
+    if (e == hipSuccess && block_split) {
+        // the sub-matrix of the copied blocks: same block rows, the copies numbered in row-major order
+        std::vector<int32_t> rp_d(mb + 1, 0), ci_d, ids;
+        ci_d.reserve((size_t)n_split_blocks);
+        ids.reserve((size_t)n_split_blocks);
+        for (size_t i = 0; i < mb; i++) {
+            for (int32_t q = row_ptr_host[i]; q < row_ptr_host[i + 1]; q++)
+                if (skip[(size_t)q]) { ci_d.push_back(p->col_idx_host[(size_t)q]); ids.push_back(q); }
+            rp_d[i + 1] = (int32_t)ci_d.size();
+        }
+        e = dev_malloc(&p->d_vals_dense, ids.size() * 256 * sizeof(uint16_t));
+        if (e == hipSuccess) e = copy_blocks(vals, ids.data(), ids.size(), p->d_vals_dense);
+        if (e == hipSuccess) {
+            SweepPlanHost h;
+            build_sweep_plan(rp_d.data(), ci_d.data(), mb, p->K / 16, h, nullptr, 0);
+            e = p->sweep_blocks.upload(h);
+        }
+        p->n_blocks_split = n_split_blocks;
+        p->n_blocks_dense = n_split_blocks;
+    } else if (e == hipSuccess && dense_sweep) {
         SweepPlanHost h;
         build_sweep_plan(row_ptr_host, p->col_idx_host.data(), mb, p->K / 16, h, dense_list.data(), dense_list.size());
         e = p->sweep_dense.upload(h);
@@ -593,7 +679,7 @@ static int smat_plan_attach_values_impl(smat_plan *p, const uint16_t *vals, cons
         return fail(e);
     }
     p->compact = c;
-    p->kernel = mixed ? SMAT_KERNEL_MIXED : SMAT_KERNEL_COMPACT;
+    p->kernel = mixed || block_split ? SMAT_KERNEL_MIXED : SMAT_KERNEL_COMPACT;
     if (p->d_bpack && want == SMAT_KERNEL_AUTO && !mixed) { // the row-wise kernel's scratch is not needed any more
         (void)dev_free(p->d_bpack);
         p->d_bpack = nullptr;
@@ -622,6 +708,8 @@ extern "C" int smat_plan_destroy(smat_plan *p)
     if (p->d_bpack) (void)dev_free(p->d_bpack);
     p->sweep.release();
     p->sweep_dense.release();
+    p->sweep_blocks.release();
+    if (p->d_vals_dense) (void)dev_free(p->d_vals_dense);
     delete p;
     return SMAT_OK;
 }
@@ -659,12 +747,14 @@ extern "C" int smat_plan_info(const smat_plan *p, int64_t *info)
     info[0] = p->kernel; info[1] = p->n_items; info[2] = p->n_split_rows; info[3] = p->chunk;
     info[4] = (int64_t)p->workspace_bytes;
     info[5] = p->kernel == SMAT_KERNEL_SWEEP ? 16 * SWEEP_TN : 16 * p->panel_tiles;
-    info[6] = p->sweep.n_ops + p->sweep_dense.n_ops; info[7] = p->sweep.n_records + p->sweep_dense.n_records;
+    info[6] = p->sweep.n_ops + p->sweep_dense.n_ops + p->sweep_blocks.n_ops;
+    info[7] = p->sweep.n_records + p->sweep_dense.n_records + p->sweep_blocks.n_records;
     info[8] = (p->d_bpack ? (int64_t)(p->K * p->n_cap * sizeof(uint16_t)) : 0) +
               (p->d_bt ? (int64_t)p->bt_bytes() : 0) +
               (p->d_bcol ? (int64_t)(p->K * p->n_cap * sizeof(uint16_t)) : 0);
     info[9] = p->compact ? p->compact->n_cols : 0;
-    info[10] = p->n_items_dense; info[11] = p->n_blocks_dense;
+    info[10] = p->sweep_blocks.d_ops ? -1 : p->n_items_dense; // -1: the mixed plan splits per block, not per block row
+    info[11] = p->n_blocks_dense;
     return SMAT_OK;
 }
 

@@ -157,6 +157,27 @@ __global__ void row_offsets_kernel(const int32_t *__restrict__ row_ptr, const in
     raw[br] = p < nnzb ? offset[p] : (nnzb ? offset[nnzb - 1] + count[nnzb - 1] : 0);
 }
 
+// Blocks that another kernel multiplies (per-block split of a mixed plan): no listed columns.
+__global__ void drop_blocks_kernel(const uint8_t *__restrict__ skip, long nnzb, uint16_t *__restrict__ mask, int32_t *__restrict__ count)
+{
+    const long p = (long)blockIdx.x * blockDim.x + threadIdx.x;
+    if (p < nnzb && skip[p]) {
+        mask[p] = 0;
+        count[p] = 0;
+    }
+}
+
+// out[j] = block ids[j] of vals (512 bytes each; 32 lanes x 16 bytes per block).
+__global__ __launch_bounds__(256) void copy_blocks_kernel(const uint16_t *__restrict__ vals, const int32_t *__restrict__ ids, long n,
+                                                          uint16_t *__restrict__ out)
+{
+    const long t = (long)blockIdx.x * blockDim.x + threadIdx.x;
+    const long j = t >> 5;
+    if (j >= n) return;
+    const int piece = (int)(t & 31);
+    reinterpret_cast<u32x4 *>(out + j * 256)[piece] = reinterpret_cast<const u32x4 *>(vals + (long)ids[j] * 256)[piece];
+}
+
 // ---- B: column-major -> row-major ----
 // 64 n x 64 k tile through LDS.  A thread reads 16 bytes (8 k) of two neighbouring columns, pairs
 // the values of equal k into dwords and writes them to the transposed tile; then every thread
@@ -201,7 +222,9 @@ __global__ __launch_bounds__(256) void transpose_b_kernel(const uint16_t *__rest
 
 // ---- the product ----
 
-template <int TQ, bool C_F32>
+// C_ACC: the result is added to what C holds (the per-block split of a mixed plan: a dense kernel has written the
+// part of the blocks it multiplies); work items that go through the workspace are not made for such plans.
+template <int TQ, bool C_F32, bool C_ACC>
 __global__ __launch_bounds__(256) void spmm_compact_kernel(
     const uint16_t *__restrict__ acol, const int32_t *__restrict__ cols, const uint16_t *__restrict__ Bt,
     void *__restrict__ Cout, float *__restrict__ workspace, const WorkItem *__restrict__ items, int n_items, int N,
@@ -399,16 +422,26 @@ __global__ __launch_bounds__(256) void spmm_compact_kernel(
                                       : reinterpret_cast<float *>(Cout) + m * (long)N;
 #pragma unroll
                 for (int h = 0; h < 8; h++)
-                    if (c0 + 4 * h < N)
-                        *reinterpret_cast<f32x4 *>(row + c0 + 4 * h) = (f32x4){o[4 * h], o[4 * h + 1], o[4 * h + 2], o[4 * h + 3]};
+                    if (c0 + 4 * h < N) {
+                        f32x4 v = {o[4 * h], o[4 * h + 1], o[4 * h + 2], o[4 * h + 3]};
+                        if (C_ACC && dst < 0) v += *reinterpret_cast<const f32x4 *>(row + c0 + 4 * h);
+                        *reinterpret_cast<f32x4 *>(row + c0 + 4 * h) = v;
+                    }
             } else {
                 uint16_t *row = reinterpret_cast<uint16_t *>(Cout) + m * (long)N;
 #pragma unroll
                 for (int h = 0; h < 4; h++) {
+                    if (c0 + 8 * h >= N) continue;
                     f16x8 v;
+                    if (C_ACC) {
+                        const f16x8 old = *reinterpret_cast<const f16x8 *>(row + c0 + 8 * h);
 #pragma unroll
-                    for (int j = 0; j < 8; j++) v[j] = (_Float16)o[8 * h + j];
-                    if (c0 + 8 * h < N) *reinterpret_cast<f16x8 *>(row + c0 + 8 * h) = v;
+                        for (int j = 0; j < 8; j++) v[j] = (_Float16)(o[8 * h + j] + (float)old[j]);
+                    } else {
+#pragma unroll
+                        for (int j = 0; j < 8; j++) v[j] = (_Float16)o[8 * h + j];
+                    }
+                    *reinterpret_cast<f16x8 *>(row + c0 + 8 * h) = v;
                 }
             }
         }
@@ -433,16 +466,26 @@ __global__ __launch_bounds__(256) void spmm_compact_kernel(
                                   : reinterpret_cast<float *>(Cout) + m * (long)N;
 #pragma unroll
             for (int h = 0; h < 4; h++)
-                if (c0 + 4 * h < N)
-                    *reinterpret_cast<f32x4 *>(row + c0 + 4 * h) = (f32x4){o[4 * h], o[4 * h + 1], o[4 * h + 2], o[4 * h + 3]};
+                if (c0 + 4 * h < N) {
+                    f32x4 v = {o[4 * h], o[4 * h + 1], o[4 * h + 2], o[4 * h + 3]};
+                    if (C_ACC && dst < 0) v += *reinterpret_cast<const f32x4 *>(row + c0 + 4 * h);
+                    *reinterpret_cast<f32x4 *>(row + c0 + 4 * h) = v;
+                }
         } else {
             uint16_t *row = reinterpret_cast<uint16_t *>(Cout) + m * (long)N;
 #pragma unroll
             for (int h = 0; h < 2; h++) {
+                if (c0 + 8 * h >= N) continue;
                 f16x8 v;
+                if (C_ACC) {
+                    const f16x8 old = *reinterpret_cast<const f16x8 *>(row + c0 + 8 * h);
 #pragma unroll
-                for (int j = 0; j < 8; j++) v[j] = (_Float16)o[8 * h + j];
-                if (c0 + 8 * h < N) *reinterpret_cast<f16x8 *>(row + c0 + 8 * h) = v;
+                    for (int j = 0; j < 8; j++) v[j] = (_Float16)(o[8 * h + j] + (float)old[j]);
+                } else {
+#pragma unroll
+                    for (int j = 0; j < 8; j++) v[j] = (_Float16)o[8 * h + j];
+                }
+                *reinterpret_cast<f16x8 *>(row + c0 + 8 * h) = v;
             }
         }
     }
@@ -468,12 +511,16 @@ hipError_t launch_compact_tq(const CompactArgs &a, hipStream_t st)
     wgs = (wgs + 7) / 8 * 8;
     if (wgs == 0) return hipSuccess;
     if (wgs > 0x7fffffffL) return hipErrorInvalidValue;
-    if (a.c_f32)
-        hipLaunchKernelGGL((spmm_compact_kernel<TQ, true>), dim3((unsigned)wgs), dim3(256), 0, st, p.d_acol, p.d_cols,
-                           a.Bt, a.C, p.d_workspace, p.d_items, p.n_items, (int)a.N, n_panels, panel_stride, row_stride);
-    else
-        hipLaunchKernelGGL((spmm_compact_kernel<TQ, false>), dim3((unsigned)wgs), dim3(256), 0, st, p.d_acol, p.d_cols,
-                           a.Bt, a.C, p.d_workspace, p.d_items, p.n_items, (int)a.N, n_panels, panel_stride, row_stride);
+    if (a.accumulate && p.n_split_rows > 0) return hipErrorInvalidValue; // partial tiles through the workspace overwrite C
+#define SMAT_LAUNCH_COMPACT(F32, ACC)                                                                                           \
+    hipLaunchKernelGGL((spmm_compact_kernel<TQ, F32, ACC>), dim3((unsigned)wgs), dim3(256), 0, st, p.d_acol, p.d_cols, a.Bt, a.C, \
+                       p.d_workspace, p.d_items, p.n_items, (int)a.N, n_panels, panel_stride, row_stride)
+    if (a.c_f32) {
+        if (a.accumulate) SMAT_LAUNCH_COMPACT(true, true); else SMAT_LAUNCH_COMPACT(true, false);
+    } else {
+        if (a.accumulate) SMAT_LAUNCH_COMPACT(false, true); else SMAT_LAUNCH_COMPACT(false, false);
+    }
+#undef SMAT_LAUNCH_COMPACT
     return hipGetLastError();
 }
 
@@ -551,9 +598,23 @@ void compact_destroy(CompactPlan *p)
     delete p;
 }
 
+hipError_t copy_blocks(const uint16_t *vals, const int32_t *ids_host, size_t n, uint16_t *out)
+{
+    if (!n) return hipSuccess;
+    Scratch ids;
+    hipError_t e = ids.alloc(n * sizeof(int32_t));
+    if (e == hipSuccess) e = hipMemcpy(ids.p, ids_host, n * sizeof(int32_t), hipMemcpyHostToDevice);
+    if (e != hipSuccess) return e;
+    hipLaunchKernelGGL(copy_blocks_kernel, dim3((unsigned)((n * 32 + 255) / 256)), dim3(256), 0, 0, vals, (const int32_t *)ids.p, (long)n, out);
+    e = hipGetLastError();
+    if (e == hipSuccess) e = hipDeviceSynchronize(); // ids goes out of scope
+    return e;
+}
+
 hipError_t compact_build(const uint16_t *vals, const int32_t *row_ptr, const int32_t *col_idx,
                          const int32_t *row_ptr_host, size_t mb, size_t nnzb, size_t n_cap, double dense_share,
-                         std::vector<uint8_t> *dense_rows, CompactPlan **out)
+                         std::vector<uint8_t> *dense_rows, CompactPlan **out, const uint8_t *skip_blocks_host,
+                         std::vector<uint8_t> *block_cols)
 {
     *out = nullptr;
     CompactPlan *p = new (std::nothrow) CompactPlan();
@@ -575,6 +636,23 @@ hipError_t compact_build(const uint16_t *vals, const int32_t *row_ptr, const int
         hipLaunchKernelGGL(colmask_kernel, dim3((unsigned)((waves + 3) / 4)), dim3(256), 0, 0, vals, (long)nnzb,
                            (uint16_t *)mask.p, (int32_t *)count.p);
         e = hipGetLastError();
+        if (block_cols) { // nonzero columns of every block, for the caller's choice of a split
+            std::vector<int32_t> cnt(nnzb);
+            SMAT_STEP(hipMemcpy(cnt.data(), count.p, nnzb * 4, hipMemcpyDeviceToHost));
+            block_cols->resize(nnzb);
+            for (size_t i = 0; i < nnzb; i++) (*block_cols)[i] = (uint8_t)cnt[i];
+        }
+        if (skip_blocks_host && e == hipSuccess) {
+            Scratch skip;
+            SMAT_STEP(skip.alloc(nnzb));
+            SMAT_STEP(hipMemcpy(skip.p, skip_blocks_host, nnzb, hipMemcpyHostToDevice));
+            if (e == hipSuccess) {
+                hipLaunchKernelGGL(drop_blocks_kernel, dim3((unsigned)((nnzb + 255) / 256)), dim3(256), 0, 0, (const uint8_t *)skip.p,
+                                   (long)nnzb, (uint16_t *)mask.p, (int32_t *)count.p);
+                e = hipGetLastError();
+            }
+            SMAT_STEP(hipDeviceSynchronize()); // skip goes out of scope
+        }
         size_t bytes = 0;
         SMAT_STEP(hipcub::DeviceScan::ExclusiveSum(nullptr, bytes, (int32_t *)count.p, (int32_t *)offset.p, (int)nnzb));
         SMAT_STEP(tmp.alloc(bytes));

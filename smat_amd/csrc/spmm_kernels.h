@@ -81,9 +81,14 @@ struct CompactPlan {
 // vals / row_ptr / col_idx: device BCSR arrays; row_ptr_host: host copy of row_ptr.
 // dense_rows != NULL and dense_share > 0: block rows with at least that share of nonzero columns get no list and no
 // work item (a dense kernel multiplies them); *dense_rows receives one flag per block row.
+// skip_blocks_host != NULL: one flag per block; flagged blocks get no listed columns (another kernel multiplies them).
+// block_cols != NULL: receives the number of nonzero columns of every block.
 hipError_t compact_build(const uint16_t *vals, const int32_t *row_ptr, const int32_t *col_idx,
                          const int32_t *row_ptr_host, size_t mb, size_t nnzb, size_t n_cap, double dense_share,
-                         std::vector<uint8_t> *dense_rows, CompactPlan **out);
+                         std::vector<uint8_t> *dense_rows, CompactPlan **out, const uint8_t *skip_blocks_host = nullptr,
+                         std::vector<uint8_t> *block_cols = nullptr);
+// out[j * 256 ..] = block ids_host[j] of vals (device to device, synchronous).
+hipError_t copy_blocks(const uint16_t *vals, const int32_t *ids_host, size_t n, uint16_t *out);
 void compact_destroy(CompactPlan *p);
 // Order-independent checksum of nnzb * 256 block values on the device (synchronous, one pass over vals).
 hipError_t values_checksum(const uint16_t *vals, size_t nnzb, uint64_t *out);
@@ -95,6 +100,7 @@ struct CompactArgs {
     size_t M, N, K;
     bool c_f32;
     const CompactPlan *plan;
+    bool accumulate = false; // C += A B instead of C = A B (plans without split rows only)
 };
 hipError_t launch_compact(const CompactArgs &a, hipStream_t st);
 hipError_t launch_b_to_col_major(const uint16_t *B_row_major, uint16_t *out, size_t N, size_t K, hipStream_t st);

@@ -148,6 +148,28 @@ def half_pruned_half_er(M=8192, keep=0.10, density=0.001, seed=0x5A170006):
             "dense_blocks": t_end}
 
 
+def pruned_plus_er(M=8192, keep=0.10, density=0.001, seed=0x5A170007):
+    """Every block row holds both kinds of blocks: the dense 16x16 blocks of block_pruned, and between them the
+    blocks of an Erdos-Renyi matrix (about one nonzero each; where one falls on a dense block the dense block stays).
+    BCSR arrays like block_pruned, plus "dense_blocks"."""
+    from . import host
+    mb = M // 16
+    top = block_pruned(M, keep, 0.02, seed)
+    er = erdos_renyi(M, density, seed ^ 0x77)
+    low = host.csr_to_bcsr(er["M"], er["K"], er["row_ptr"], er["col_idx"], er["val"])
+    key_d = np.repeat(np.arange(mb, dtype=np.int64), np.diff(top["b_row_ptr"])) * mb + top["b_col_idx"].astype(np.int64) // 16
+    key_s = np.repeat(np.arange(mb, dtype=np.int64), np.diff(low.row_ptr)) * mb + low.col_idx.astype(np.int64) // 16
+    only_s = ~np.isin(key_s, key_d)
+    keys = np.concatenate([key_d, key_s[only_s]])
+    vals = np.concatenate([np.asarray(top["b_val"]).reshape(-1, 256), np.asarray(low.val).reshape(-1, 256)[only_s]])
+    order = np.argsort(keys, kind="stable")
+    keys, vals = keys[order], vals[order]
+    row_ptr = np.zeros(mb + 1, np.int64)
+    np.add.at(row_ptr, keys // mb + 1, 1)
+    return {"M": M, "K": M, "b_row_ptr": np.cumsum(row_ptr).astype(np.int32), "b_col_idx": ((keys % mb) * 16).astype(np.int32),
+            "b_val": np.ascontiguousarray(vals).ravel(), "nnzb": int(keys.size), "dense_blocks": int(key_d.size)}
+
+
 def bcsr_to_csr(M, b_row_ptr, b_col_idx, b_val, drop_zeros=False):
     """Expands BCSR blocks to a CSR (all 256 entries per block unless drop_zeros)."""
     mb = M // 16

@@ -194,6 +194,45 @@ def test_mixed_dispatch_full_size(smat, cuda, oracle):
     check_sampled(oracle, A, B, N, C, sample_rows(mb, 16, extra=(mb // 2 - 1, mb // 2, mb // 2 + 1)))
 
 
+def test_mixed_dispatch_per_block(smat, cuda, oracle):
+    """4096 x 4096, every block row holds dense blocks (10 % of the grid) and blocks of about one nonzero between them,
+    N = 4096: no block row is of one kind, so the plan splits per BLOCK - a copy of the dense blocks through the sweep
+    kernel, the columns of the other blocks added by the compact kernel - and the result is the product of the
+    whole matrix (fp16 and fp32 C; row-major B; the same split when asked for by name)."""
+    import torch
+    A = gen.pruned_plus_er(4096, 0.10, 0.003)
+    N = 4096
+    M, K, nnzb = A["M"], A["K"], A["nnzb"]
+    B = gen.dense_b(K, N, seed=0xB0000007, dist="normal")
+    C, info = gpu_spmm_compact(smat, cuda, A, B, N, kernel=0)
+    assert info["kernel"] == 6 and info["mixed_dense_items"] == -1      # mixed, per block
+    assert info["mixed_dense_blocks"] == A["dense_blocks"] and info["sweep_ops"] > 0
+    assert 0 < info["compact_cols"] < 3 * (nnzb - A["dense_blocks"])     # the list holds the other blocks only
+    mb = M // 16
+    rows = sample_rows(mb, 24, extra=(0, 1, 63, 64, mb - 1))
+    check_sampled(oracle, A, B, N, C, rows)
+    C6, info6 = gpu_spmm_compact(smat, cuda, A, B, N, kernel=6)
+    assert info6["mixed_dense_items"] == -1 and np.array_equal(C6, C)
+    # fp32 C: only the summation order differs from one kernel over the whole matrix
+    C32, _ = gpu_spmm_compact(smat, cuda, A, B, N, kernel=0, c_f32=True)
+    C32_one, info_one = gpu_spmm_compact(smat, cuda, A, B, N, kernel=2, c_f32=True)
+    assert info_one["kernel"] == 2
+    scale = np.sqrt((C32_one.astype(np.float64) ** 2).sum(axis=1)).max()
+    assert np.abs(C32 - C32_one).max() <= 2e-6 * scale
+    # the same through row-major B (the sweep kernel takes it from the plan's column-major copy, the compact kernel in place)
+    B_rm = np.ascontiguousarray(B.reshape(N, K).T).ravel()
+    vals, rp, ci = (to_dev(torch, A["b_val"], cuda), to_dev(torch, A["b_row_ptr"].astype(np.int32), cuda),
+                    to_dev(torch, A["b_col_idx"].astype(np.int32), cuda))
+    p = smat.Plan(A["b_row_ptr"], M, K, nnzb, N, col_idx_host=A["b_col_idx"], kernel=0, b_row_major=True)
+    p.attach_values(vals, rp, ci)
+    assert p.info()["mixed_dense_items"] == -1
+    Cd = torch.full((M, N), 0x7E00, dtype=torch.int16, device=cuda)
+    smat.spmm(vals, rp, ci, to_dev(torch, B_rm, cuda), Cd, M, N, K, nnzb, plan=p, b_row_major=True)
+    torch.cuda.synchronize()
+    p.close()
+    assert np.array_equal(Cd.cpu().numpy().view(np.uint16), C)
+
+
 def test_config4_sweep_kernel_full_size_linearity_and_more_rows(smat, cuda, oracle):
     """Headline config through the plan's choice (the sweep kernel): 40 sampled block rows against the oracle
     (first and last of every row group among them), and A (2 B) = 2 (A B) bit for bit over the whole result."""
