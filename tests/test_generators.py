@@ -55,3 +55,21 @@ def test_stencil_values():
     v = d["val"].view(np.float16).astype(np.float32)
     assert (v[rows == d["col_idx"]] == 26).all() and (v[rows != d["col_idx"]] == -1).all()
     assert d["row_ptr"][-1] == 10 ** 3  # (3n-2)^3
+
+
+def test_pruned_plus_er_holds_both_kinds_of_blocks_in_every_row():
+    A = gen.pruned_plus_er(2048, 0.10, 0.003)
+    top = gen.block_pruned(2048, 0.10, 0.02, 0x5A170007)
+    mb = 128
+    rp, ci = A["b_row_ptr"], A["b_col_idx"]
+    assert A["dense_blocks"] == top["nnzb"] and A["nnzb"] > 2 * top["nnzb"] and rp[-1] == A["nnzb"]
+    vals = A["b_val"].reshape(-1, 256)
+    full = ((vals & 0x7FFF) != 0).sum(axis=1) > 200          # a dense block; the others hold a handful of entries
+    assert full.sum() == top["nnzb"] and ((vals[~full] & 0x7FFF) != 0).sum(axis=1).max() <= 8
+    for r in range(mb):
+        seg = ci[rp[r]:rp[r + 1]]
+        assert (np.diff(seg) > 0).all() and (seg % 16 == 0).all()
+        kinds = full[rp[r]:rp[r + 1]]
+        assert kinds.any() and (~kinds).any()                 # no block row of one kind
+        dense_cols = seg[kinds]
+        assert np.array_equal(dense_cols, top["b_col_idx"][top["b_row_ptr"][r]:top["b_row_ptr"][r + 1]])
