@@ -647,16 +647,24 @@ static int smat_plan_attach_values_impl(smat_plan *p, const uint16_t *vals, cons
         e = dev_malloc(&p->d_vals_dense, ids.size() * 256 * sizeof(uint16_t));
         if (e == hipSuccess) e = copy_blocks(vals, ids.data(), ids.size(), p->d_vals_dense);
         if (e == hipSuccess) {
-            SweepPlanHost h;
-            build_sweep_plan(rp_d.data(), ci_d.data(), mb, p->K / 16, h, nullptr, 0);
-            e = p->sweep_blocks.upload(h);
+            try { // the list and the copies made so far are released by fail() below
+                SweepPlanHost h;
+                build_sweep_plan(rp_d.data(), ci_d.data(), mb, p->K / 16, h, nullptr, 0);
+                e = p->sweep_blocks.upload(h);
+            } catch (...) {
+                e = hipErrorOutOfMemory;
+            }
         }
         p->n_blocks_split = n_split_blocks;
         p->n_blocks_dense = n_split_blocks;
     } else if (e == hipSuccess && dense_sweep) {
-        SweepPlanHost h;
-        build_sweep_plan(row_ptr_host, p->col_idx_host.data(), mb, p->K / 16, h, dense_list.data(), dense_list.size());
-        e = p->sweep_dense.upload(h);
+        try {
+            SweepPlanHost h;
+            build_sweep_plan(row_ptr_host, p->col_idx_host.data(), mb, p->K / 16, h, dense_list.data(), dense_list.size());
+            e = p->sweep_dense.upload(h);
+        } catch (...) {
+            e = hipErrorOutOfMemory;
+        }
         p->n_blocks_dense = blocks_dense;
     } else if (e == hipSuccess && mixed) {
         std::vector<WorkItem> items;
