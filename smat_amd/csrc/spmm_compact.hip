@@ -62,6 +62,7 @@ typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
 
 namespace {
 
+int g_force_run = 0;
 int g_force_tq = 0; // test hook: 1 or 2 = panels of 64 or 128 columns whatever the sizes say, 0 = the launcher decides
 
 constexpr int LIST_PAD = 640; // entries readable past the end of the list (the index loads of the 64-column panel run up to 16 steps ahead)
@@ -228,15 +229,20 @@ template <int TQ, bool C_F32, bool C_ACC>
 __global__ __launch_bounds__(256) void spmm_compact_kernel(
     const uint16_t *__restrict__ acol, const int32_t *__restrict__ cols, const uint16_t *__restrict__ Bt,
     void *__restrict__ Cout, float *__restrict__ workspace, const WorkItem *__restrict__ items, int n_items, int N,
-    int n_panels, long panel_stride, long row_stride)
+    int n_panels, long panel_stride, long row_stride, unsigned xcd_run)
 {
     constexpr int PANEL = 64 * TQ;
     const int lane = threadIdx.x & 63;
     const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
-    // panel-major order of the (panel, item) space, a contiguous eighth per XCD
+    // Panel-major order of the (panel, item) space.  An XCD gets the workgroup ids that are equal modulo 8, whatever
+    // their work costs; here the XCDs take runs of xcd_run consecutive workgroups of that order in turn (gridDim.x is a
+    // multiple of 8 * xcd_run).  One run per XCD keeps neighbouring block rows, which share rows of B, on one L2;
+    // short runs even out a list whose cost per item changes along it (R-MAT: 60 to 70 % of the steps are in the first
+    // quarter of the items, and the launch took as long as the XCD that got them).
     const long total = (long)n_items * n_panels;
-    const int chunk = gridDim.x >> 3; // gridDim.x is a multiple of 8
-    const long wg = (long)(blockIdx.x & 7) * chunk + (blockIdx.x >> 3);
+    const unsigned slot = blockIdx.x >> 3;
+    const unsigned run = __builtin_amdgcn_readfirstlane(slot / xcd_run);
+    const long wg = ((long)run * 8 + (blockIdx.x & 7)) * xcd_run + (slot - run * xcd_run);
     const long w = wg * 4 + wave;
     if (w >= total) return;
     const int panel = (int)(w / n_items);
@@ -508,13 +514,15 @@ hipError_t launch_compact_tq(const CompactArgs &a, hipStream_t st)
     }
     const long total = (long)p.n_items * n_panels;
     long wgs = (total + 3) / 4;
-    wgs = (wgs + 7) / 8 * 8;
     if (wgs == 0) return hipSuccess;
+    long xcd_run = compact_xcd_run(p, n_panels);
+    if (g_force_run > 0) xcd_run = std::min<long>((wgs + 7) / 8, g_force_run);
+    wgs = (wgs + 8 * xcd_run - 1) / (8 * xcd_run) * (8 * xcd_run);
     if (wgs > 0x7fffffffL) return hipErrorInvalidValue;
     if (a.accumulate && p.n_split_rows > 0) return hipErrorInvalidValue; // partial tiles through the workspace overwrite C
 #define SMAT_LAUNCH_COMPACT(F32, ACC)                                                                                           \
     hipLaunchKernelGGL((spmm_compact_kernel<TQ, F32, ACC>), dim3((unsigned)wgs), dim3(256), 0, st, p.d_acol, p.d_cols, a.Bt, a.C, \
-                       p.d_workspace, p.d_items, p.n_items, (int)a.N, n_panels, panel_stride, row_stride)
+                       p.d_workspace, p.d_items, p.n_items, (int)a.N, n_panels, panel_stride, row_stride, (unsigned)xcd_run)
     if (a.c_f32) {
         if (a.accumulate) SMAT_LAUNCH_COMPACT(true, true); else SMAT_LAUNCH_COMPACT(true, false);
     } else {
@@ -564,6 +572,43 @@ hipError_t launch_compact(const CompactArgs &a_in, hipStream_t st)
     if (a.plan->n_split_rows > 0)
         e = launch_reduce(a.plan->d_workspace, a.plan->d_split, a.plan->n_split_rows, a.C, a.N, a.c_f32, st);
     return e;
+}
+
+unsigned choose_xcd_run(const uint64_t *P, uint64_t n, int n_panels)
+{
+    const uint64_t total = n * (uint64_t)n_panels;
+    const uint64_t wgs = (total + 3) / 4;
+    const uint64_t eighth = std::max<uint64_t>((wgs + 7) / 8, 1);
+    if (n == 0 || P[n] == 0) return (unsigned)eighth;
+    auto cost_before = [&](uint64_t wg) { // of the workgroups before wg in the panel-major item space
+        const uint64_t w = std::min(wg * 4, total);
+        return (w / n) * P[n] + P[w % n];
+    };
+    uint64_t best_run = eighth;
+    double best = 1e30;
+    for (uint64_t run : {eighth, (uint64_t)1024, (uint64_t)256, (uint64_t)64, (uint64_t)16, (uint64_t)4}) {
+        if (run > eighth || (run == eighth && best < 1e30)) continue;
+        uint64_t load[8] = {0, 0, 0, 0, 0, 0, 0, 0};
+        for (uint64_t first = 0, x = 0; first < wgs; first += run, x = (x + 1) & 7)
+            load[x] += cost_before(first + run) - cost_before(first);
+        const uint64_t busiest = *std::max_element(load, load + 8);
+        const double ratio = (double)busiest * 8.0 / (double)std::max<uint64_t>(cost_before(wgs), 1);
+        if (ratio < best) best = ratio, best_run = run;
+        if (ratio <= 1.04) break;
+    }
+    return (unsigned)best_run;
+}
+
+unsigned compact_xcd_run(const CompactPlan &p, int n_panels)
+{
+    const uint64_t n = (uint64_t)p.n_items;
+    if (p.cost_prefix.size() != n + 1) return (unsigned)std::max<uint64_t>(((n * (uint64_t)n_panels + 3) / 4 + 7) / 8, 1);
+    std::lock_guard<std::mutex> lock(p.run_mutex);
+    for (const auto &known : p.xcd_runs)
+        if (known.first == n_panels) return known.second;
+    const unsigned run = choose_xcd_run(p.cost_prefix.data(), n, n_panels);
+    p.xcd_runs.emplace_back(n_panels, run);
+    return run;
 }
 
 hipError_t values_checksum(const uint16_t *vals, size_t nnzb, uint64_t *out)
@@ -729,6 +774,11 @@ hipError_t compact_build(const uint16_t *vals, const int32_t *row_ptr, const int
         items.push_back(WorkItem{(int32_t)i, cc_host[i], cc_host[i + 1], -1});
     }
     if (dense_rows) *dense_rows = dense;
+    // what an item costs, for the deal of the items to the XCDs: its steps, and two more for fetching the item, the
+    // first indices and the stores of its tile
+    p->cost_prefix.assign(items.size() + 1, 0);
+    for (size_t i = 0; i < items.size(); i++)
+        p->cost_prefix[i + 1] = p->cost_prefix[i] + (uint64_t)((items[i].end - items[i].begin + 31) / 32) + 2;
     p->n_items = (int)items.size();
     p->n_split_rows = (int)split.size();
     p->n_slots = slot;
@@ -755,3 +805,10 @@ hipError_t compact_build(const uint16_t *vals, const int32_t *row_ptr, const int
 // Test hook (not part of smat.h): 1 or 2 = the compact kernel works on panels of 64 or 128 columns whatever the sizes
 // say (each width has its own way of gathering the rows of B), 0 = the launcher decides (the default).
 extern "C" void smat_internal_compact_panel(int tq) { smat::g_force_tq = tq; }
+// Test hooks for the deal of the compact kernel's workgroups to the XCDs: a run length that every launch uses
+// (0 = chosen per plan and number of panels), and the choice itself for a list of item costs (host only).
+extern "C" void smat_internal_compact_run(int run) { smat::g_force_run = run; }
+extern "C" unsigned smat_internal_choose_xcd_run(const uint64_t *cost_prefix, uint64_t n_items, int n_panels)
+{
+    return smat::choose_xcd_run(cost_prefix, n_items, n_panels);
+}

@@ -3,6 +3,8 @@
 #include <hip/hip_runtime.h>
 
 #include "sweep_format.h"
+#include <mutex>
+#include <utility>
 #include <vector>
 #include <stddef.h>
 #include <stdint.h>
@@ -77,7 +79,18 @@ struct CompactPlan {
     int64_t n_cols = 0;           // nonzero block columns listed (without padding)
     int64_t n_cols_all = 0;       // nonzero block columns of the whole matrix
     uint64_t values_checksum = 0; // of the block values the lists were made from
+    // How the launch deals the work items to the XCDs: cost_prefix[i] = estimated cost (steps of 32 columns plus a
+    // constant per item) of the items before item i; xcd_runs caches the run length chosen for a number of panels.
+    std::vector<uint64_t> cost_prefix;
+    mutable std::mutex run_mutex;
+    mutable std::vector<std::pair<int, unsigned>> xcd_runs;
 };
+// Workgroups per run for a launch of n_panels panels: the XCDs take runs of that many consecutive workgroups
+// (4 work items each, panel-major) in turn.  The longest run that keeps the estimated load of the busiest XCD
+// within 4 % of the mean, a contiguous eighth of the launch if that does.
+unsigned compact_xcd_run(const CompactPlan &p, int n_panels);
+// The choice itself: cost_prefix[i] = cost of the items before item i (n_items + 1 entries).
+unsigned choose_xcd_run(const uint64_t *cost_prefix, uint64_t n_items, int n_panels);
 // vals / row_ptr / col_idx: device BCSR arrays; row_ptr_host: host copy of row_ptr.
 // dense_rows != NULL and dense_share > 0: block rows with at least that share of nonzero columns get no list and no
 // work item (a dense kernel multiplies them); *dense_rows receives one flag per block row.

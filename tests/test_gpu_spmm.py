@@ -771,6 +771,34 @@ def test_compact_kernel_power_law_rows(smat, cuda, oracle):
     assert np.array_equal(C32 * np.float32(2), C32_2)
 
 
+def test_compact_kernel_same_bits_however_the_items_are_dealt_to_the_xcds(smat, cuda, oracle):
+    """The launch deals its workgroups to the XCDs in runs whose length it picks from the cost of the items (one
+    run per XCD where that is balanced, short runs on lists like this one, R-MAT with its long block rows first).
+    The deal decides where an item runs, never what it computes: every run length gives the bits of the launcher's
+    own choice, on 1, 2 and 5 panels, with the split rows' partial tiles, and with a grid that the rounding to whole
+    runs makes larger than the work."""
+    import ctypes as C_
+    lib = smat.lib
+    lib.smat_internal_compact_run.argtypes, lib.smat_internal_compact_run.restype = [C_.c_int], None
+    d = gen.rmat(14, 16, seed=33)
+    A = bcsr_of(smat, d)
+    rows = np.repeat(np.arange(d["M"], dtype=np.int64), np.diff(d["row_ptr"]))
+    per_row = np.bincount(np.unique((rows // 16) * d["K"] + d["col_idx"]) // d["K"])   # nonzero columns per block row
+    assert per_row.max() > max(4 * per_row[per_row > 0].mean(), 512) + 32                # some block row is split
+    try:
+        for N in (64, 128, 264):
+            B = gen.dense_b(A["K"], N, seed=N + 1, dist="uniform")
+            lib.smat_internal_compact_run(0)
+            C, _ = gpu_spmm_compact(smat, cuda, A, B, N)
+            assert oracle.compare(C, oracle_ref(oracle, A, B, N))[0] <= TOL_F16
+            for run in (1, 3, 4, 16, 50, 64, 256, 1 << 20):
+                lib.smat_internal_compact_run(run)
+                C_run, _ = gpu_spmm_compact(smat, cuda, A, B, N)
+                assert np.array_equal(C_run, C), (N, run)
+    finally:
+        lib.smat_internal_compact_run(0)
+
+
 def test_plan_check_tells_patterns_apart(smat, cuda):
     """Two matrices of the same M, K and nnzb: the launch cannot tell them apart, smat_plan_check can."""
     A = gen.random_bcsr(20, 24, 0.25, seed=41)
