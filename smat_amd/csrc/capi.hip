@@ -68,6 +68,7 @@ struct smat_plan {
     uint16_t *d_bt = nullptr; // copy of B in panels of rows, K * (n_cap rounded up to 256) halves (compact kernel)
     size_t bt_bytes() const { return K * ((n_cap + 255) / 256 * 256) * sizeof(uint16_t); }
     // mixed dispatch (after smat_plan_attach_values): row-wise work list of the block rows with mostly full blocks
+    XcdDeal deal, deal_dense; // of d_items and d_items_dense; cost of an item: its pairs of blocks, and two more
     WorkItem *d_items_dense = nullptr;
     SplitRow *d_split_dense = nullptr;
     float *d_workspace_dense = nullptr;
@@ -176,6 +177,7 @@ extern "C" int smat_spmm_bcsr_f16_ex(const uint16_t *vals, const int32_t *row_pt
         a.workspace = plan->d_workspace;
         a.panel_tiles = plan->panel_tiles;
         a.max_item_blocks = plan->max_item_blocks;
+        a.deal = &plan->deal;
         if (plan->d_bpack && N <= plan->n_cap && o.kernel != SMAT_KERNEL_ROWWISE_DIRECT) a.b_packed = plan->d_bpack;
     }
     int kernel = o.kernel;
@@ -230,6 +232,7 @@ extern "C" int smat_spmm_bcsr_f16_ex(const uint16_t *vals, const int32_t *row_pt
             d.split_rows = plan->d_split_dense; d.n_split_rows = plan->n_split_dense;
             d.workspace = plan->d_workspace_dense;
             d.max_item_blocks = 0; // describes the whole matrix's list, not this one
+            d.deal = &plan->deal_dense;
             e = d.n_items ? launch_rowwise(d, static_cast<hipStream_t>(o.stream)) : hipSuccess;
         }
         if (e == hipSuccess) {
@@ -329,6 +332,14 @@ static uint64_t pattern_fingerprint(const int32_t *row_ptr_host, const int32_t *
 
 // Row-wise work list: whole block rows, rows longer than `chunk` blocks in chunks with a partial-sum slot each
 // (split rows first: they are the longest items).  only != NULL: just the block rows it flags.  Returns the slots.
+static void rowwise_costs(const std::vector<WorkItem> &items, XcdDeal &deal)
+{
+    std::vector<uint64_t> prefix(items.size() + 1, 0);
+    for (size_t i = 0; i < items.size(); i++)
+        prefix[i + 1] = prefix[i] + (uint64_t)((items[i].end - items[i].begin + 1) / 2) + 2;
+    deal.set_costs(std::move(prefix));
+}
+
 static int rowwise_work_list(const int32_t *row_ptr_host, size_t mb, long chunk, const uint8_t *only,
                              std::vector<WorkItem> &items, std::vector<SplitRow> &split)
 {
@@ -423,6 +434,7 @@ static int smat_plan_create_impl(smat_plan **out, const int32_t *row_ptr_host,
     std::vector<SplitRow> split;
     const int slot = rowwise_work_list(row_ptr_host, mb, chunk, nullptr, items, split);
     p->n_items = (int)items.size();
+    rowwise_costs(items, p->deal);
     for (const WorkItem &wi : items) p->max_item_blocks = std::max(p->max_item_blocks, wi.end - wi.begin);
     p->panel_tiles = rowwise_panel_tiles(n_hint, 0, items.size());
     p->n_split_rows = (int)split.size();
@@ -671,6 +683,7 @@ static int smat_plan_attach_values_impl(smat_plan *p, const uint16_t *vals, cons
         std::vector<SplitRow> split;
         const int slots = rowwise_work_list(row_ptr_host, mb, p->chunk, dense.data(), items, split);
         p->n_items_dense = (int)items.size();
+        rowwise_costs(items, p->deal_dense);
         p->n_split_dense = (int)split.size();
         p->n_blocks_dense = blocks_dense;
         e = dev_malloc(&p->d_items_dense, std::max<size_t>(items.size(), 1) * sizeof(WorkItem));

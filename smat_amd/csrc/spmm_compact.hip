@@ -63,6 +63,7 @@ typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
 namespace {
 
 int g_force_run = 0;
+int g_last_run = 0; // test hook: the run length of the latest launch
 int g_force_tq = 0; // test hook: 1 or 2 = panels of 64 or 128 columns whatever the sizes say, 0 = the launcher decides
 
 constexpr int LIST_PAD = 640; // entries readable past the end of the list (the index loads of the 64-column panel run up to 16 steps ahead)
@@ -515,8 +516,9 @@ hipError_t launch_compact_tq(const CompactArgs &a, hipStream_t st)
     const long total = (long)p.n_items * n_panels;
     long wgs = (total + 3) / 4;
     if (wgs == 0) return hipSuccess;
-    long xcd_run = compact_xcd_run(p, n_panels);
+    long xcd_run = p.deal.run((size_t)p.n_items, n_panels);
     if (g_force_run > 0) xcd_run = std::min<long>((wgs + 7) / 8, g_force_run);
+    g_last_run = (int)xcd_run;
     wgs = (wgs + 8 * xcd_run - 1) / (8 * xcd_run) * (8 * xcd_run);
     if (wgs > 0x7fffffffL) return hipErrorInvalidValue;
     if (a.accumulate && p.n_split_rows > 0) return hipErrorInvalidValue; // partial tiles through the workspace overwrite C
@@ -572,43 +574,6 @@ hipError_t launch_compact(const CompactArgs &a_in, hipStream_t st)
     if (a.plan->n_split_rows > 0)
         e = launch_reduce(a.plan->d_workspace, a.plan->d_split, a.plan->n_split_rows, a.C, a.N, a.c_f32, st);
     return e;
-}
-
-unsigned choose_xcd_run(const uint64_t *P, uint64_t n, int n_panels)
-{
-    const uint64_t total = n * (uint64_t)n_panels;
-    const uint64_t wgs = (total + 3) / 4;
-    const uint64_t eighth = std::max<uint64_t>((wgs + 7) / 8, 1);
-    if (n == 0 || P[n] == 0) return (unsigned)eighth;
-    auto cost_before = [&](uint64_t wg) { // of the workgroups before wg in the panel-major item space
-        const uint64_t w = std::min(wg * 4, total);
-        return (w / n) * P[n] + P[w % n];
-    };
-    uint64_t best_run = eighth;
-    double best = 1e30;
-    for (uint64_t run : {eighth, (uint64_t)1024, (uint64_t)256, (uint64_t)64, (uint64_t)16, (uint64_t)4}) {
-        if (run > eighth || (run == eighth && best < 1e30)) continue;
-        uint64_t load[8] = {0, 0, 0, 0, 0, 0, 0, 0};
-        for (uint64_t first = 0, x = 0; first < wgs; first += run, x = (x + 1) & 7)
-            load[x] += cost_before(first + run) - cost_before(first);
-        const uint64_t busiest = *std::max_element(load, load + 8);
-        const double ratio = (double)busiest * 8.0 / (double)std::max<uint64_t>(cost_before(wgs), 1);
-        if (ratio < best) best = ratio, best_run = run;
-        if (ratio <= 1.04) break;
-    }
-    return (unsigned)best_run;
-}
-
-unsigned compact_xcd_run(const CompactPlan &p, int n_panels)
-{
-    const uint64_t n = (uint64_t)p.n_items;
-    if (p.cost_prefix.size() != n + 1) return (unsigned)std::max<uint64_t>(((n * (uint64_t)n_panels + 3) / 4 + 7) / 8, 1);
-    std::lock_guard<std::mutex> lock(p.run_mutex);
-    for (const auto &known : p.xcd_runs)
-        if (known.first == n_panels) return known.second;
-    const unsigned run = choose_xcd_run(p.cost_prefix.data(), n, n_panels);
-    p.xcd_runs.emplace_back(n_panels, run);
-    return run;
 }
 
 hipError_t values_checksum(const uint16_t *vals, size_t nnzb, uint64_t *out)
@@ -776,9 +741,10 @@ hipError_t compact_build(const uint16_t *vals, const int32_t *row_ptr, const int
     if (dense_rows) *dense_rows = dense;
     // what an item costs, for the deal of the items to the XCDs: its steps, and two more for fetching the item, the
     // first indices and the stores of its tile
-    p->cost_prefix.assign(items.size() + 1, 0);
+    std::vector<uint64_t> cost_prefix(items.size() + 1, 0);
     for (size_t i = 0; i < items.size(); i++)
-        p->cost_prefix[i + 1] = p->cost_prefix[i] + (uint64_t)((items[i].end - items[i].begin + 31) / 32) + 2;
+        cost_prefix[i + 1] = cost_prefix[i] + (uint64_t)((items[i].end - items[i].begin + 31) / 32) + 2;
+    p->deal.set_costs(std::move(cost_prefix));
     p->n_items = (int)items.size();
     p->n_split_rows = (int)split.size();
     p->n_slots = slot;
@@ -806,8 +772,10 @@ hipError_t compact_build(const uint16_t *vals, const int32_t *row_ptr, const int
 // say (each width has its own way of gathering the rows of B), 0 = the launcher decides (the default).
 extern "C" void smat_internal_compact_panel(int tq) { smat::g_force_tq = tq; }
 // Test hooks for the deal of the compact kernel's workgroups to the XCDs: a run length that every launch uses
-// (0 = chosen per plan and number of panels), and the choice itself for a list of item costs (host only).
+// (0 = chosen per plan and number of panels), the run length of the latest launch, and the choice itself for a list
+// of item costs (host only).
 extern "C" void smat_internal_compact_run(int run) { smat::g_force_run = run; }
+extern "C" int smat_internal_compact_last_run(void) { return smat::g_last_run; }
 extern "C" unsigned smat_internal_choose_xcd_run(const uint64_t *cost_prefix, uint64_t n_items, int n_panels)
 {
     return smat::choose_xcd_run(cost_prefix, n_items, n_panels);

@@ -28,6 +28,26 @@ struct SplitRow {
     int32_t pad;
 };
 
+// How a launch over a work list deals its workgroups to the eight XCDs.  The dispatcher gives an XCD the workgroup
+// ids that are equal modulo 8, whatever their work costs; the row-wise and the compact kernel lay the panel-major
+// (panel, item) space (4 items per workgroup) out in runs of consecutive workgroups that the XCDs take in turn.
+// One run per XCD keeps neighbouring block rows, which share rows of B, on one L2; short runs even out a list whose
+// cost per item changes along it.
+// choose_xcd_run: the longest run among {an eighth of the launch, 1024, 256, 64, 16, 4} that keeps the estimated load
+// of the busiest XCD within 4 % of the mean (the best of them if none does); cost_prefix[i] = cost of the items
+// before item i (n_items + 1 entries).
+unsigned choose_xcd_run(const uint64_t *cost_prefix, uint64_t n_items, int n_panels);
+struct XcdDeal {
+    void set_costs(std::vector<uint64_t> &&prefix); // of another list: forgets the choices made for the old one
+    // the choice for a launch of n_items x n_panels (kept once made); an eighth of the launch if the costs are not
+    // those of a list of n_items
+    unsigned run(size_t n_items, int n_panels) const;
+private:
+    std::vector<uint64_t> cost_prefix_;
+    mutable std::mutex mutex_;
+    mutable std::vector<std::pair<int, unsigned>> known_;
+};
+
 struct SpmmArgs {
     const uint16_t *vals;
     const int32_t *row_ptr;
@@ -44,6 +64,7 @@ struct SpmmArgs {
     float *workspace; // device, n_slots * 16 * N floats
     uint16_t *b_packed; // device scratch of K * N halves, or nullptr: read the column-major B directly
     int max_item_blocks; // blocks of the longest work item, 0 = not known (no plan): lets short rows take the short-row kernel
+    const XcdDeal *deal; // how to deal the items to the XCDs; nullptr = an eighth of the launch each
 };
 
 // Stream format and geometry of the sweep kernel: sweep_format.h (shared with the host-side plan builder).
@@ -79,18 +100,8 @@ struct CompactPlan {
     int64_t n_cols = 0;           // nonzero block columns listed (without padding)
     int64_t n_cols_all = 0;       // nonzero block columns of the whole matrix
     uint64_t values_checksum = 0; // of the block values the lists were made from
-    // How the launch deals the work items to the XCDs: cost_prefix[i] = estimated cost (steps of 32 columns plus a
-    // constant per item) of the items before item i; xcd_runs caches the run length chosen for a number of panels.
-    std::vector<uint64_t> cost_prefix;
-    mutable std::mutex run_mutex;
-    mutable std::vector<std::pair<int, unsigned>> xcd_runs;
+    XcdDeal deal;                 // cost of an item: its steps of 32 columns, and two more
 };
-// Workgroups per run for a launch of n_panels panels: the XCDs take runs of that many consecutive workgroups
-// (4 work items each, panel-major) in turn.  The longest run that keeps the estimated load of the busiest XCD
-// within 4 % of the mean, a contiguous eighth of the launch if that does.
-unsigned compact_xcd_run(const CompactPlan &p, int n_panels);
-// The choice itself: cost_prefix[i] = cost of the items before item i (n_items + 1 entries).
-unsigned choose_xcd_run(const uint64_t *cost_prefix, uint64_t n_items, int n_panels);
 // vals / row_ptr / col_idx: device BCSR arrays; row_ptr_host: host copy of row_ptr.
 // dense_rows != NULL and dense_share > 0: block rows with at least that share of nonzero columns get no list and no
 // work item (a dense kernel multiplies them); *dense_rows receives one flag per block row.

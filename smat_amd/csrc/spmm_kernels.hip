@@ -19,6 +19,8 @@
 #include <hip/hip_runtime.h>
 #include <stdint.h>
 
+#include <algorithm>
+
 #include "spmm_kernels.h"
 
 #define SMAT_ORDER_FENCE()                      \
@@ -63,8 +65,10 @@ __device__ __forceinline__ int ncol_of(int t, int i)
 // Item index runs fastest inside a panel, so the four wavefronts of a workgroup
 // and neighbouring workgroups share one B panel (K x 16*TN) in L2.  Workgroup
 // ids are dealt round-robin to the 8 XCDs by the dispatcher; the remap below
-// gives each XCD a contiguous eighth of the (panel-major) item space so that an
-// XCD's private L2 holds few distinct B panels.
+// gives the XCDs runs of xcd_run consecutive workgroups of the (panel-major) item
+// space in turn: an eighth of the launch each, so that an XCD's private L2 holds few
+// distinct B panels, or shorter runs where the items' cost changes along the list
+// (gridDim.x is a multiple of 8 * xcd_run).
 // amdgpu_waves_per_eu(1, 4): at most 4 wavefronts per SIMD are asked for, which leaves the
 // compiler 128 registers; with the default target of 8 it squeezes the kernel into 64 and
 // gets there by loading each operand right before its MFMA, one memory latency apiece.
@@ -77,7 +81,7 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 4))) voi
     const uint16_t *__restrict__ vals, const int32_t *__restrict__ row_ptr,
     const int32_t *__restrict__ col_idx, const uint16_t *__restrict__ B, void *__restrict__ Cout,
     float *__restrict__ workspace, const WorkItem *__restrict__ items, int n_items, int N, long K,
-    int n_panels)
+    int n_panels, unsigned xcd_run)
 {
     constexpr int TG = TN < 4 ? TN : 4;
     constexpr int PANEL = 16 * TN;
@@ -86,8 +90,9 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 4))) voi
     const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
 
     const long total = (long)n_items * n_panels;
-    const int chunk = gridDim.x >> 3; // gridDim.x is a multiple of 8
-    const long wg = (long)(blockIdx.x & 7) * chunk + (blockIdx.x >> 3);
+    const unsigned slot = blockIdx.x >> 3;
+    const unsigned run = __builtin_amdgcn_readfirstlane(slot / xcd_run);
+    const long wg = ((long)run * 8 + (blockIdx.x & 7)) * xcd_run + (slot - run * xcd_run);
     const long w = wg * 4 + wave;
     if (w >= total) return;
     const int panel = (int)(w / n_items);
@@ -382,14 +387,15 @@ static hipError_t launch_rowwise_tn(const SpmmArgs &a, hipStream_t st)
     const int n_panels = (int)((a.N + panel - 1) / panel);
     const long total = (long)a.n_items * n_panels;
     long wgs = (total + 3) / 4;
-    wgs = (wgs + 7) / 8 * 8;
     if (wgs == 0) return hipSuccess;
+    const long xcd_run = a.deal && a.items ? (long)a.deal->run((size_t)a.n_items, n_panels) : (wgs + 7) / 8;
+    wgs = (wgs + 8 * xcd_run - 1) / (8 * xcd_run) * (8 * xcd_run);
     if (wgs > 0x7fffffffL) return hipErrorInvalidValue;
     dim3 grid((unsigned)wgs), block(256);
 #define SMAT_LAUNCH_ROWWISE(F32, PK)                                                              \
     hipLaunchKernelGGL((spmm_rowwise_kernel<TN, F32, PK>), grid, block, 0, st, a.vals, a.row_ptr, \
                        a.col_idx, a.b_packed ? a.b_packed : a.B, a.C, a.workspace, a.items,       \
-                       a.n_items, (int)a.N, (long)a.K, n_panels)
+                       a.n_items, (int)a.N, (long)a.K, n_panels, (unsigned)xcd_run)
     if (a.b_packed) {
         if (a.c_f32) SMAT_LAUNCH_ROWWISE(true, true);
         else SMAT_LAUNCH_ROWWISE(false, true);
@@ -399,6 +405,51 @@ static hipError_t launch_rowwise_tn(const SpmmArgs &a, hipStream_t st)
     }
 #undef SMAT_LAUNCH_ROWWISE
     return hipGetLastError();
+}
+
+unsigned choose_xcd_run(const uint64_t *P, uint64_t n, int n_panels)
+{
+    const uint64_t total = n * (uint64_t)n_panels;
+    const uint64_t wgs = (total + 3) / 4;
+    const uint64_t eighth = std::max<uint64_t>((wgs + 7) / 8, 1);
+    if (n == 0 || P[n] == 0) return (unsigned)eighth;
+    auto cost_before = [&](uint64_t wg) { // of the workgroups before wg in the panel-major item space
+        const uint64_t w = std::min(wg * 4, total);
+        return (w / n) * P[n] + P[w % n];
+    };
+    uint64_t best_run = eighth;
+    double best = 1e30;
+    for (uint64_t run : {eighth, (uint64_t)1024, (uint64_t)256, (uint64_t)64, (uint64_t)16, (uint64_t)4}) {
+        if (run > eighth || (run == eighth && best < 1e30)) continue;
+        uint64_t load[8] = {0, 0, 0, 0, 0, 0, 0, 0};
+        for (uint64_t first = 0, x = 0; first < wgs; first += run, x = (x + 1) & 7)
+            load[x] += cost_before(first + run) - cost_before(first);
+        const uint64_t busiest = *std::max_element(load, load + 8);
+        const double ratio = (double)busiest * 8.0 / (double)std::max<uint64_t>(cost_before(wgs), 1);
+        if (ratio < best) best = ratio, best_run = run;
+        if (ratio <= 1.04) break;
+    }
+    return (unsigned)best_run;
+}
+
+void XcdDeal::set_costs(std::vector<uint64_t> &&prefix)
+{
+    std::lock_guard<std::mutex> lock(mutex_);
+    cost_prefix_ = std::move(prefix);
+    known_.clear();
+}
+
+unsigned XcdDeal::run(size_t n_items, int n_panels) const
+{
+    const uint64_t n = n_items;
+    std::lock_guard<std::mutex> lock(mutex_);
+    if (n == 0 || cost_prefix_.size() != n + 1) // no costs for this list: an eighth of the launch each
+        return (unsigned)std::max<uint64_t>(((n * (uint64_t)n_panels + 3) / 4 + 7) / 8, 1);
+    for (const auto &k : known_)
+        if (k.first == n_panels) return k.second;
+    const unsigned r = choose_xcd_run(cost_prefix_.data(), n, n_panels);
+    known_.emplace_back(n_panels, r);
+    return r;
 }
 
 int rowwise_panel_tiles(size_t N, int requested, size_t n_items)

@@ -113,6 +113,9 @@ def test_config3_rmat_scale20_reordered_full_size(smat, cuda, oracle):
     C2 = torch.full((M, N), 0x7E00, dtype=torch.int16, device=cuda)
     smat.spmm(vals, rp, ci, B2d, C2, M, N, K, nnzb, plan=plan)
     torch.cuda.synchronize()
+    # the long block rows are at the front of the list: the launch deals its workgroups to the XCDs in short runs
+    # (one run per XCD would be about 4,400 workgroups and leave one XCD with most of the steps)
+    assert 0 < smat.lib.smat_internal_compact_last_run() <= 64
     plan.close()
     C_host = C.cpu().numpy().view(np.uint16)
     check_sampled(oracle, A, B, N, C_host, rows)

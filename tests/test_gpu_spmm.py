@@ -267,6 +267,40 @@ def test_skewed_rows_with_and_without_plan(smat, cuda, oracle, lengths):
     assert rel_err_f32(c32, ref) <= TOL_F32
 
 
+@pytest.mark.parametrize("kernel", [3, 4])
+def test_rowwise_kernel_power_law_rows_dealt_in_short_runs(smat, cuda, oracle, kernel):
+    """R-MAT scale 14 through the row-wise kernel with a plan (B read in place, and from the slab-major copy): the
+    list has the chunks of the long block rows first, and one run of workgroups per XCD would give the first XCD
+    several times the mean, so the launch deals them in short runs.  1, 2 and 4 panels; the fp16 result carries the
+    bits of the fp32 one rounded once."""
+    import ctypes as C_
+    d = gen.rmat(14, 16, seed=34)
+    A = bcsr_of(smat, d)
+    lens = np.diff(A["b_row_ptr"]).astype(np.int64)
+    avg = lens[lens > 0].mean()
+    chunk = (max(int(4.0 * avg + 0.5), 64) + 1) & ~1
+    assert lens.max() > 2 * chunk                                   # some block row is split
+    # the list as the plan builds it (chunks of the split rows, then the other rows), at two more than its pairs per item
+    split = [min(chunk, n - b) for n in lens[lens > chunk] for b in range(0, n, chunk)]
+    costs = np.array(split + list(lens[lens <= chunk]), np.uint64)
+    costs = (costs + np.uint64(1)) // np.uint64(2) + np.uint64(2)
+    prefix = np.concatenate([[0], np.cumsum(costs)]).astype(np.uint64)
+    choose = smat.lib.smat_internal_choose_xcd_run
+    choose.restype, choose.argtypes = C_.c_uint, [C_.c_void_p, C_.c_uint64, C_.c_int]
+    for N in (64, 128, 256):
+        n_panels = N // 64
+        eighth = ((len(costs) * n_panels + 3) // 4 + 7) // 8
+        if n_panels < 4:
+            assert choose(prefix.ctypes.data, len(costs), n_panels) < eighth
+        B = gen.dense_b(A["K"], N, seed=N + 3, dist="uniform")
+        ref = oracle_ref(oracle, A, B, N)
+        C = gpu_spmm(smat, cuda, A, B, N, plan=True, kernel=kernel)
+        assert oracle.compare(C, ref)[0] <= TOL_F16
+        C32 = gpu_spmm(smat, cuda, A, B, N, plan=True, kernel=kernel, c_f32=True)
+        assert rel_err_f32(C32, ref) <= TOL_F32
+        assert np.array_equal(C32.astype(np.float16).view(np.uint16), C)
+
+
 @pytest.mark.parametrize("N", [32, 40, 64, 88, 128, 264])
 def test_short_rows_with_a_plan_match_the_oracle_and_the_general_kernel(smat, cuda, oracle, N):
     """Rows of 0..10 blocks with a plan: the launcher takes the kernel that loads all operands of a row at once.
