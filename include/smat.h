@@ -152,7 +152,10 @@ int smat_plan_create(smat_plan **plan, const int32_t *row_ptr_host, const int32_
  * SMAT_KERNEL_AUTO the plan switches to that kernel when fewer than 60% of the block columns
  * are nonzero.  The compact kernel works from the copy: attach again after the values change.
  * The new list is built before the old one is dropped; if the call fails the plan has no list and
- * SMAT_KERNEL_AUTO goes back to the sweep or row-wise kernel.  Synchronous.  No counterpart in the reference, which multiplies every block as a dense
+ * SMAT_KERNEL_AUTO goes back to the sweep or row-wise kernel.  When the plan takes the compact kernel, the call also
+ * times a few launches of it on zeros (temporary device buffers of K x n_hint and M x n_hint halves, freed before it
+ * returns; skipped if they do not fit) to choose how the work is dealt to the GPU's eight XCDs: a choice that moves
+ * no bit of any result.  Synchronous.  No counterpart in the reference, which multiplies every block as a dense
  * 16x16 (mmaCBT.cu:44-66). */
 int smat_plan_attach_values(smat_plan *plan, const uint16_t *vals, const int32_t *row_ptr,
                             const int32_t *col_idx, const int32_t *row_ptr_host);

@@ -701,6 +701,10 @@ static int smat_plan_attach_values_impl(smat_plan *p, const uint16_t *vals, cons
     }
     p->compact = c;
     p->kernel = mixed || block_split ? SMAT_KERNEL_MIXED : SMAT_KERNEL_COMPACT;
+    // the deal of the compact kernel's work items to the XCDs, measured on this list at the plan's width (B in the
+    // layout the plan was made for: d_bcol is the scratch of a plan for row-major B)
+    e = compact_tune(*c, p->d_bt, p->M, p->n_cap, p->K, p->d_bcol != nullptr, block_split);
+    if (e != hipSuccess) return set_error(SMAT_ERR_HIP, "timing the compact kernel failed: %s", hipGetErrorString(e));
     if (p->d_bpack && want == SMAT_KERNEL_AUTO && !mixed) { // the row-wise kernel's scratch is not needed any more
         (void)dev_free(p->d_bpack);
         p->d_bpack = nullptr;

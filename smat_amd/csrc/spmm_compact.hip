@@ -63,6 +63,7 @@ typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
 namespace {
 
 int g_force_run = 0;
+int g_tune = 1; // test hook: 0 = attaching values measures nothing, the estimate decides the deal
 int g_last_run = 0; // test hook: the run length of the latest launch
 int g_force_tq = 0; // test hook: 1 or 2 = panels of 64 or 128 columns whatever the sizes say, 0 = the launcher decides
 
@@ -517,7 +518,10 @@ hipError_t launch_compact_tq(const CompactArgs &a, hipStream_t st)
     long wgs = (total + 3) / 4;
     if (wgs == 0) return hipSuccess;
     long xcd_run = p.deal.run((size_t)p.n_items, n_panels);
-    if (g_force_run > 0) xcd_run = std::min<long>((wgs + 7) / 8, g_force_run);
+    if (p.tuned_run > 0 && p.tuned_n == a.N) xcd_run = p.tuned_run;
+    if (a.xcd_run > 0) xcd_run = a.xcd_run;
+    if (g_force_run > 0) xcd_run = g_force_run;
+    xcd_run = std::min<long>((wgs + 7) / 8, xcd_run);
     g_last_run = (int)xcd_run;
     wgs = (wgs + 8 * xcd_run - 1) / (8 * xcd_run) * (8 * xcd_run);
     if (wgs > 0x7fffffffL) return hipErrorInvalidValue;
@@ -551,6 +555,17 @@ hipError_t launch_b_to_col_major(const uint16_t *B_row_major, uint16_t *out, siz
     return hipGetLastError();
 }
 
+// The panel width of a launch, in units of 64 columns.
+static int compact_panel_width(const CompactPlan &p, size_t N, size_t K)
+{
+    const long items = p.n_items;
+    int tq = 1;
+    if (N >= 128 && items * (long)(N / 128) >= 2048 && p.n_cols >= (int64_t)items * 384) tq = 2;
+    if (g_force_tq == 1 || g_force_tq == 2) tq = g_force_tq;
+    while (tq > 1 && K * (size_t)(64 * tq) * sizeof(uint16_t) > ((size_t)128 << 20)) tq >>= 1;
+    return tq;
+}
+
 hipError_t launch_compact(const CompactArgs &a_in, hipStream_t st)
 {
     CompactArgs a = a_in;
@@ -563,16 +578,70 @@ hipError_t launch_compact(const CompactArgs &a_in, hipStream_t st)
     // rows of B that the gathers hit at random come from one panel at a time: a panel is kept under half of the
     // 256 MiB memory-side cache (the lists of A and the rows of C stream through it too).  On a 2^20-row B at
     // N = 128 the panel of 64 columns (128 MiB) takes 0.74 x the time of the panel of 128.
-    const long items = a.plan->n_items;
-    int tq = 1;
-    if (a.N >= 128 && items * (long)(a.N / 128) >= 2048 && a.plan->n_cols >= (int64_t)items * 384) tq = 2;
-    if (g_force_tq == 1 || g_force_tq == 2) tq = g_force_tq;
-    while (tq > 1 && a.K * (size_t)(64 * tq) * sizeof(uint16_t) > ((size_t)128 << 20)) tq >>= 1;
+    const int tq = compact_panel_width(*a.plan, a.N, a.K);
     if (tq == 2) e = launch_compact_tq<2>(a, st);
     else e = launch_compact_tq<1>(a, st);
     if (e != hipSuccess) return e;
     if (a.plan->n_split_rows > 0)
         e = launch_reduce(a.plan->d_workspace, a.plan->d_split, a.plan->n_split_rows, a.C, a.N, a.c_f32, st);
+    return e;
+}
+
+hipError_t compact_tune(CompactPlan &p, uint16_t *Bt, size_t M, size_t N, size_t K, bool b_row_major, bool accumulate)
+{
+    p.tuned_n = 0;
+    p.tuned_run = 0;
+    if (!g_tune || p.n_items == 0 || N == 0 || !Bt) return hipSuccess;
+    Scratch B, C;
+    if (B.alloc(K * N * sizeof(uint16_t)) != hipSuccess || C.alloc(M * N * sizeof(uint16_t)) != hipSuccess) {
+        (void)hipGetLastError(); // no room for the trial: not an error of the plan
+        return hipSuccess;
+    }
+    hipError_t e = hipMemset(B.p, 0, K * N * sizeof(uint16_t));
+    if (e == hipSuccess) e = hipMemset(C.p, 0, M * N * sizeof(uint16_t));
+    hipEvent_t t0 = nullptr, t1 = nullptr;
+    if (e == hipSuccess) e = hipEventCreate(&t0);
+    if (e == hipSuccess) e = hipEventCreate(&t1);
+    CompactArgs a{};
+    a.B = static_cast<const uint16_t *>(B.p); a.b_row_major = b_row_major; a.Bt = Bt; a.C = C.p;
+    a.M = M; a.N = N; a.K = K; a.c_f32 = false; a.plan = &p; a.accumulate = accumulate;
+    auto time_of = [&](unsigned run, int launches, float *ms) {
+        a.xcd_run = run;
+        hipError_t r = launch_compact(a, nullptr); // warm-up
+        if (r == hipSuccess) r = hipEventRecord(t0, nullptr);
+        for (int i = 0; i < launches && r == hipSuccess; i++) r = launch_compact(a, nullptr);
+        if (r == hipSuccess) r = hipEventRecord(t1, nullptr);
+        if (r == hipSuccess) r = hipEventSynchronize(t1);
+        if (r == hipSuccess) r = hipEventElapsedTime(ms, t0, t1);
+        *ms /= (float)launches;
+        return r;
+    };
+    // the run length of an untuned launch, as launch_compact_tq computes it for this N
+    const int tq = compact_panel_width(p, N, K);
+    const int n_panels = (int)((N + 64 * tq - 1) / (64 * tq));
+    const long wgs = ((long)p.n_items * n_panels + 3) / 4;
+    const unsigned eighth = (unsigned)std::max<long>((wgs + 7) / 8, 1);
+    const unsigned base = std::min(eighth, p.deal.run((size_t)p.n_items, n_panels));
+    float t_base = 0.f;
+    if (e == hipSuccess) e = time_of(base, 1, &t_base);
+    if (e == hipSuccess && t_base <= 20.f) {
+        std::vector<unsigned> runs{base};
+        if (base * 4 >= eighth) // a list that the estimate finds even: the longer runs are worth a try
+            for (unsigned r : {eighth, eighth / 2, eighth / 4})
+                if (r >= 4 && std::find(runs.begin(), runs.end(), r) == runs.end()) runs.push_back(r);
+        const int launches = t_base < 0.2f ? 20 : t_base < 2.f ? 6 : 3;
+        unsigned best_run = base;
+        float best = 0.f;
+        for (size_t i = 0; i < runs.size() && e == hipSuccess; i++) {
+            float ms = 0.f;
+            e = time_of(runs[i], launches, &ms);
+            if (i == 0) best = ms * 0.97f; // another run length has to be 3 % faster than the estimate's choice
+            else if (ms < best) best = ms, best_run = runs[i];
+        }
+        if (e == hipSuccess) p.tuned_n = N, p.tuned_run = best_run;
+    }
+    if (t0) (void)hipEventDestroy(t0);
+    if (t1) (void)hipEventDestroy(t1);
     return e;
 }
 
@@ -776,6 +845,7 @@ extern "C" void smat_internal_compact_panel(int tq) { smat::g_force_tq = tq; }
 // of item costs (host only).
 extern "C" void smat_internal_compact_run(int run) { smat::g_force_run = run; }
 extern "C" int smat_internal_compact_last_run(void) { return smat::g_last_run; }
+extern "C" void smat_internal_compact_tune(int on) { smat::g_tune = on; }
 extern "C" unsigned smat_internal_choose_xcd_run(const uint64_t *cost_prefix, uint64_t n_items, int n_panels)
 {
     return smat::choose_xcd_run(cost_prefix, n_items, n_panels);

@@ -101,6 +101,10 @@ struct CompactPlan {
     int64_t n_cols_all = 0;       // nonzero block columns of the whole matrix
     uint64_t values_checksum = 0; // of the block values the lists were made from
     XcdDeal deal;                 // cost of an item: its steps of 32 columns, and two more
+    // Measured once, when the values are attached (compact_tune): the run length of the deal to the XCDs for
+    // launches of tuned_n columns; 0 = not measured, the estimate from the costs decides.
+    size_t tuned_n = 0;
+    unsigned tuned_run = 0;
 };
 // vals / row_ptr / col_idx: device BCSR arrays; row_ptr_host: host copy of row_ptr.
 // dense_rows != NULL and dense_share > 0: block rows with at least that share of nonzero columns get no list and no
@@ -123,10 +127,17 @@ struct CompactArgs {
     void *C;
     size_t M, N, K;
     bool c_f32;
+    unsigned xcd_run = 0; // 0 = the plan's choice
     const CompactPlan *plan;
     bool accumulate = false; // C += A B instead of C = A B (plans without split rows only)
 };
 hipError_t launch_compact(const CompactArgs &a, hipStream_t st);
+// Times launches of M x N x K with a few run lengths of the deal to the XCDs (the estimate's choice, an eighth of the
+// launch, a half and a quarter of that) on zeros in temporary buffers and keeps the fastest for launches of N columns
+// (tuned_n, tuned_run).  The deal decides where an item runs, not what it computes: the results do not depend on
+// it.  Synchronous, default stream; a plan too large for the temporary buffers, or whose single launch takes
+// longer than 20 ms, keeps the estimate's choice.
+hipError_t compact_tune(CompactPlan &p, uint16_t *Bt, size_t M, size_t N, size_t K, bool b_row_major, bool accumulate);
 hipError_t launch_b_to_col_major(const uint16_t *B_row_major, uint16_t *out, size_t N, size_t K, hipStream_t st);
 
 int rowwise_panel_tiles(size_t N, int requested, size_t n_items);

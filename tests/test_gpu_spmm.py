@@ -833,6 +833,38 @@ def test_compact_kernel_same_bits_however_the_items_are_dealt_to_the_xcds(smat, 
         lib.smat_internal_compact_run(0)
 
 
+def test_attaching_values_times_the_deal_and_the_result_does_not_depend_on_it(smat, cuda, oracle):
+    """smat_plan_attach_values times a few launches on zeros with different run lengths of the deal to the XCDs and
+    keeps the fastest for launches at the plan's width.  Whatever it keeps is one of its candidates (the estimate's
+    choice, an eighth of the launch, a half or a quarter of that), other widths go by the estimate, and the bits are
+    those of a plan that measured nothing."""
+    import ctypes as C_
+    lib = smat.lib
+    lib.smat_internal_compact_tune.argtypes, lib.smat_internal_compact_tune.restype = [C_.c_int], None
+    lib.smat_internal_compact_last_run.restype = C_.c_int
+    A = bcsr_of(smat, gen.erdos_renyi(4096, 0.004, seed=79))    # 256 block rows of about 16 steps
+    n_items = A["M"] // 16
+    try:
+        for n_hint, N in ((256, 256), (512, 512), (512, 264)):
+            B = gen.dense_b(A["K"], N, seed=N + 11, dist="normal")
+            lib.smat_internal_compact_tune(0)
+            C_plain, _ = gpu_spmm_compact(smat, cuda, A, B, N, n_hint=n_hint)
+            run_plain = lib.smat_internal_compact_last_run()
+            lib.smat_internal_compact_tune(1)
+            C_timed, _ = gpu_spmm_compact(smat, cuda, A, B, N, n_hint=n_hint)
+            run_timed = lib.smat_internal_compact_last_run()
+            assert np.array_equal(C_timed, C_plain)
+            assert oracle.compare(C_timed, oracle_ref(oracle, A, B, N))[0] <= TOL_F16
+            eighth = ((n_items * ((N + 63) // 64) + 3) // 4 + 7) // 8
+            assert run_plain == eighth                           # rows of one length: one run per XCD by the estimate
+            if N == n_hint:
+                assert run_timed in (eighth, eighth // 2, eighth // 4)
+            else:
+                assert run_timed == run_plain                    # measured for 512 columns, launched with 264
+    finally:
+        lib.smat_internal_compact_tune(1)
+
+
 def test_plan_check_tells_patterns_apart(smat, cuda):
     """Two matrices of the same M, K and nnzb: the launch cannot tell them apart, smat_plan_check can."""
     A = gen.random_bcsr(20, 24, 0.25, seed=41)
