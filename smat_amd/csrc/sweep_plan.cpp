@@ -4,6 +4,9 @@
 #include <algorithm>
 #include <cstdlib>
 #include <cstring>
+#include <functional>
+#include <queue>
+#include <utility>
 
 #include <stdexcept>
 
@@ -23,8 +26,48 @@ void build_sweep_plan(const int32_t *row_ptr, const int32_t *col_idx, size_t mb,
                       const int32_t *rows, size_t n_rows)
 {
     if (!rows) n_rows = mb;
-    auto row_at = [&](size_t i) { return rows ? (size_t)rows[i] : i; }; // i-th block row of the plan
     const size_t n_rg = (n_rows + G - 1) / G;
+    // Row groups: G block rows of the list each, in list order - unless that leaves one group with far more blocks
+    // than the average.  A workgroup multiplies one row group under several panels, so the launch takes as long as
+    // the heaviest group; then the rows are dealt out instead: in descending block count, each to the group with the
+    // fewest blocks so far that still has room (the group sizes stay what they were).  Which rows share a group
+    // matters for nothing else: the rows of C are found through row_map, and a matrix dense enough for this kernel
+    // touches every K chunk from any 64 of its rows.
+    std::vector<int32_t> order;
+    {
+        std::vector<int64_t> blocks_of(n_rg, 0);
+        int64_t total = 0, heaviest = 0;
+        for (size_t i = 0; i < n_rows; i++) {
+            const size_t br = rows ? (size_t)rows[i] : i;
+            blocks_of[i / G] += row_ptr[br + 1] - row_ptr[br];
+        }
+        for (size_t rg = 0; rg < n_rg; rg++) total += blocks_of[rg], heaviest = std::max(heaviest, blocks_of[rg]);
+        if (n_rg > 1 && (double)heaviest * (double)n_rows > 1.08 * (double)total * (double)G) {
+            std::vector<int32_t> by_count(n_rows);
+            for (size_t i = 0; i < n_rows; i++) by_count[i] = rows ? rows[i] : (int32_t)i;
+            std::stable_sort(by_count.begin(), by_count.end(), [&](int32_t x, int32_t y) {
+                return row_ptr[x + 1] - row_ptr[x] > row_ptr[y + 1] - row_ptr[y];
+            });
+            std::vector<std::vector<int32_t>> members(n_rg);
+            typedef std::pair<int64_t, size_t> Load; // blocks so far, row group
+            std::priority_queue<Load, std::vector<Load>, std::greater<Load>> lightest;
+            for (size_t rg = 0; rg < n_rg; rg++) lightest.push(Load(0, rg));
+            for (int32_t br : by_count) {
+                const Load l = lightest.top();
+                lightest.pop();
+                const size_t rg = l.second;
+                members[rg].push_back(br);
+                if (members[rg].size() < std::min(n_rows, (rg + 1) * G) - rg * G)
+                    lightest.push(Load(l.first + (row_ptr[br + 1] - row_ptr[br]), rg));
+            }
+            order.reserve(n_rows);
+            for (size_t rg = 0; rg < n_rg; rg++) {
+                std::sort(members[rg].begin(), members[rg].end());
+                order.insert(order.end(), members[rg].begin(), members[rg].end());
+            }
+        }
+    }
+    auto row_at = [&](size_t i) { return !order.empty() ? (size_t)order[i] : rows ? (size_t)rows[i] : i; }; // i-th block row of the plan
     const size_t n_kchunks = (kb + S - 1) / S;
     const int32_t nnzb = row_ptr[mb];
     out = SweepPlanHost();

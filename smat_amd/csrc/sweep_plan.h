@@ -24,7 +24,8 @@ struct SweepPlanHost {
 
 // row_ptr / col_idx: host BCSR (col_idx = absolute first column of each block, validated by the caller);
 // at least two blocks.  rows != NULL: only these n_rows block rows (ascending) are multiplied and stored, packed
-// 64 to a row group; the others belong to another kernel.
+// 64 to a row group; the others belong to another kernel.  The rows go to the row groups in list order, or, where
+// that leaves one group with over 1.08 x the blocks of an average one, by their block count (row_map says where).
 void build_sweep_plan(const int32_t *row_ptr, const int32_t *col_idx, size_t mb, size_t kb, SweepPlanHost &out,
                       const int32_t *rows = nullptr, size_t n_rows = 0);
 

@@ -130,6 +130,26 @@ def block_pruned(M=8192, keep=0.10, sigma=0.02, seed=0x5A170004):
     return {"M": M, "K": M, "b_row_ptr": row_ptr, "b_col_idx": col_idx, "b_val": val, "nnzb": kept}
 
 
+def block_pruned_skewed(M=8192, keep_first=0.18, keep_last=0.02, sigma=0.02, seed=0x5A170008):
+    """A block-pruned weight whose rows were pruned unevenly: block row i keeps each of its blocks with a probability
+    that falls linearly from keep_first (row 0) to keep_last (last row); kept blocks dense with N(0, sigma) values
+    drawn as in block_pruned.  BCSR arrays like block_pruned."""
+    mb = M // 16
+    cells = mb * mb
+    keep = keep_first + (keep_last - keep_first) * np.arange(mb, dtype=np.float64) / max(mb - 1, 1)
+    u = (rand_u64(seed, np.arange(cells, dtype=np.uint64)) >> np.uint64(11)).astype(np.float64) * 2.0 ** -53
+    sel = np.nonzero(u < np.repeat(keep, mb))[0]
+    br, bc = sel // mb, sel % mb
+    row_ptr = np.zeros(mb + 1, dtype=np.int64)
+    np.add.at(row_ptr, br + 1, 1)
+    e = np.arange(256, dtype=np.int64)
+    rows = (br[:, None] * 16 + e[None, :] // 16)
+    cols = (bc[:, None] * 16 + e[None, :] % 16)
+    val = f16_bits(sigma * rand_normal(seed ^ 0xA5A5, (rows * M + cols).ravel()))
+    return {"M": M, "K": M, "b_row_ptr": np.cumsum(row_ptr).astype(np.int32), "b_col_idx": (bc * 16).astype(np.int32),
+            "b_val": val, "nnzb": int(sel.size)}
+
+
 def half_pruned_half_er(M=8192, keep=0.10, density=0.001, seed=0x5A170006):
     """A matrix of two kinds of rows: the upper half of its block rows from block_pruned (dense 16x16 blocks), the
     lower half the blocking of an Erdos-Renyi matrix (about one nonzero per block).  BCSR arrays like block_pruned."""

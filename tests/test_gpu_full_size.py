@@ -236,6 +236,26 @@ def test_mixed_dispatch_per_block(smat, cuda, oracle):
     assert np.array_equal(Cd.cpu().numpy().view(np.uint16), C)
 
 
+def test_sweep_kernel_unevenly_pruned_rows(smat, cuda, oracle):
+    """8192 x 8192, dense blocks whose share falls from 18 % in the first block row to 2 % in the last, N = 4096: the
+    sweep kernel's plan deals the block rows to its row groups by their block count (in order, the first group
+    would hold 1.7 x the average), so the rows of C of one workgroup are scattered over the matrix.  Sampled block rows
+    (the first and the last, the heaviest and an empty one if there is one) against the oracle, fp16 and fp32 C."""
+    A = gen.block_pruned_skewed(8192, 0.18, 0.02)
+    N = 4096
+    M, K, nnzb = A["M"], A["K"], A["nnzb"]
+    lens = np.diff(A["b_row_ptr"])
+    assert lens.reshape(-1, 64).sum(1).max() > 1.5 * lens.sum() / 8
+    B = gen.dense_b(K, N, seed=0xB0000008, dist="normal")
+    C, info = gpu_spmm_compact(smat, cuda, A, B, N, kernel=0)
+    assert info["kernel"] == 2 and info["sweep_ops"] > 0
+    mb = M // 16
+    rows = sample_rows(mb, 24, extra=(0, 1, 63, 64, mb - 1, int(np.argmax(lens)), int(np.argmin(lens))))
+    check_sampled(oracle, A, B, N, C, rows)
+    C32, _ = gpu_spmm_compact(smat, cuda, A, B, N, kernel=2, c_f32=True)
+    assert np.array_equal(C32.astype(np.float16).view(np.uint16), C)
+
+
 def test_config4_sweep_kernel_full_size_linearity_and_more_rows(smat, cuda, oracle):
     """Headline config through the plan's choice (the sweep kernel): 40 sampled block rows against the oracle
     (first and last of every row group among them), and A (2 B) = 2 (A B) bit for bit over the whole result."""

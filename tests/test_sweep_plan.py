@@ -87,8 +87,13 @@ def replay(plan, A, Bd, rows=None):
     n_rg = plan["rg_chunk_ptr"].size - 1
     n_real = n_fill = 0
     subset = np.arange(M // 16) if rows is None else np.asarray(rows)
-    place = {int(br): i for i, br in enumerate(subset)}  # block row -> position in the plan's list of rows
     row_len = np.diff(rp)
+    group_of = {}  # block row -> its row group
+    for rg in range(n_rg):
+        got = plan["row_map"][rg * G:(rg + 1) * G]
+        for b in got[got >= 0]:
+            assert int(b) not in group_of
+            group_of[int(b)] = rg
     for rg in range(n_rg):
         chunks = plan["chunk_ids"][plan["rg_chunk_ptr"][rg]:plan["rg_chunk_ptr"][rg + 1]]
         assert np.all(np.diff(chunks) > 0)
@@ -152,7 +157,7 @@ def replay(plan, A, Bd, rows=None):
                         assert q == 0
                     continue
                 n_real += 1
-                assert br in place and place[br] // G == rg
+                assert group_of.get(br) == rg
                 # both loaded blocks belong to the op's block row, also when one of them multiplies zeros: only a
                 # block that is alone in its row travels with another row's block
                 if row_len[br] >= 2:
@@ -178,9 +183,24 @@ def replay(plan, A, Bd, rows=None):
     assert n_fill == plan["fillers"] and n_real == plan["pairs"] + plan["singles"]
     mapped = plan["row_map"][plan["row_map"] >= 0]
     assert np.array_equal(np.sort(mapped), np.sort(subset)), "row_map is not a partition of the plan's block rows"
-    for rg in range(n_rg):  # row group rg holds the rows subset[64 rg : 64 rg + 64], the slots that are left say -1
-        got = plan["row_map"][rg * G:(rg + 1) * G]
-        assert np.array_equal(np.sort(got[got >= 0]), np.sort(subset[rg * G:(rg + 1) * G]))
+    # Row group rg holds the rows subset[64 rg : 64 rg + 64] (the slots that are left say -1) - unless that grouping
+    # leaves one group with more than 1.08 x the blocks of an average one: then the rows are dealt out by their block
+    # count, heaviest first to the lightest group with room, and every group keeps its size
+    groups = [plan["row_map"][rg * G:(rg + 1) * G] for rg in range(n_rg)]
+    groups = [g[g >= 0] for g in groups]
+    in_order = [row_len[subset[rg * G:(rg + 1) * G]].sum() for rg in range(n_rg)]
+    skewed = n_rg > 1 and max(in_order) * subset.size > 1.08 * sum(in_order) * G
+    plan["dealt"] = bool(skewed)
+    for rg in range(n_rg):
+        assert groups[rg].size == subset[rg * G:(rg + 1) * G].size
+        if not skewed:
+            assert np.array_equal(np.sort(groups[rg]), np.sort(subset[rg * G:(rg + 1) * G]))
+    if skewed:
+        dealt = np.array([row_len[g].sum() for g in groups])
+        full = [rg for rg in range(n_rg) if groups[rg].size == G]
+        # no full group is heavier than the lightest full group by more than one row (what dealing heaviest-first gives)
+        assert dealt[full].max() - dealt[full].min() <= row_len[subset].max()
+        assert dealt.max() <= max(in_order)
     # read-ahead: the entries after the last stream exist and are harmless
     tail = plan["ops"][plan["n_entries"]:]
     assert tail.shape[0] == PAD and np.all(tail == np.array([0, ZERO_OFF, 0, END_OFF], np.uint32))
@@ -282,6 +302,32 @@ def test_headline_matrix_pairs_nearly_everything():
     assert plan["period_max_sum"] * WAVES < 1.045 * (plan["pairs"] + plan["singles"] + plan["fillers"])
     per_wave = np.diff(plan["op_ptr"])
     assert per_wave.min() >= 4 * 32 + 1 and per_wave.max() <= 72 * 32
+
+
+def test_unevenly_pruned_rows_are_dealt_to_even_row_groups():
+    """A workgroup multiplies one row group under several panels, so a launch takes as long as its heaviest row group.
+    Block rows whose density falls from 18 % to 2 % would give the first of four groups 1.6 x the average; the plan
+    deals the rows out instead, and the streams still multiply every block once into its own rows of C."""
+    A = gen.block_pruned_skewed(4096, 0.18, 0.02)
+    lens = np.diff(A["b_row_ptr"])
+    in_order = lens.reshape(-1, G).sum(1)
+    assert in_order.max() > 1.5 * in_order.mean()
+    plan = sweep_plan(A["b_row_ptr"], A["b_col_idx"], A["M"], A["K"])
+    Bd = np.random.default_rng(3).normal(size=(A["K"], 4))
+    Cd = replay(plan, A, Bd)
+    assert plan["dealt"]
+    assert np.allclose(Cd, dense_of(A) @ Bd, rtol=1e-12, atol=1e-12)
+    dealt = np.array([lens[g[g >= 0]].sum() for g in plan["row_map"].reshape(-1, G)])
+    assert dealt.max() < 1.01 * dealt.mean()
+    # the busiest wavefront of a period still has hardly more ops than the average one
+    assert plan["period_max_sum"] * WAVES < 1.06 * (plan["pairs"] + plan["singles"] + plan["fillers"])
+
+
+def test_evenly_pruned_rows_stay_in_order():
+    A = gen.block_pruned(8192, 0.10, 0.02)
+    plan = sweep_plan(A["b_row_ptr"], A["b_col_idx"], A["M"], A["K"])
+    for rg, g in enumerate(plan["row_map"].reshape(-1, G)):
+        assert np.array_equal(np.sort(g), np.arange(rg * G, (rg + 1) * G))
 
 
 def test_committed_interpreter_loop_is_what_the_generator_writes():
