@@ -410,6 +410,10 @@ def main():
         if "mfma_busy" in prof:
             roof["mfma_busy_rocprof"] = prof["mfma_busy"]
     roof["kernel_ms"] = round(kernel_ms, 5)
+    if roof["traffic"]:
+        # the rate of the bytes that the profiled launch moved beyond the L2 (part of them served by the memory-side
+        # cache): below the algorithmic rate where a kernel does not read the zeros inside the blocks
+        roof["traffic_gbs"] = round(roof["traffic"] / (kernel_ms * 1e-3) / 1e9, 1)
     roof["kernel_ms_single_launch"] = {"n": int(singles.size), "median": round(float(np.median(singles)), 5),
                                        "min": round(float(singles.min()), 5), "max": round(float(singles.max()), 5)}
     roof["measured_mfma_peak_tflops"] = round(peak.value, 1)
