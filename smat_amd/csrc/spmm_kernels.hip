@@ -421,6 +421,7 @@ unsigned choose_xcd_run(const uint64_t *P, uint64_t n, int n_panels)
     double best = 1e30;
     for (uint64_t run : {eighth, (uint64_t)1024, (uint64_t)256, (uint64_t)64, (uint64_t)16, (uint64_t)4}) {
         if (run > eighth || (run == eighth && best < 1e30)) continue;
+        if (wgs / run > ((uint64_t)1 << 26)) break; // a launch this large is not walked run by run on the host
         uint64_t load[8] = {0, 0, 0, 0, 0, 0, 0, 0};
         for (uint64_t first = 0, x = 0; first < wgs; first += run, x = (x + 1) & 7)
             load[x] += cost_before(first + run) - cost_before(first);

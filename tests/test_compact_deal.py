@@ -98,3 +98,4 @@ def test_random_lists_agree_with_the_numpy_deal():
             assert run == first_ok or abs(ratios[cands.index(first_ok)] - LIMIT) < 1e-6 or abs(ratios[cands.index(run)] - LIMIT) < 1e-6
         else:
             assert ratios[cands.index(run)] <= min(ratios) + 1e-9
+
