@@ -131,6 +131,11 @@ def build_workload(name, want_b=True):
         # both kinds of blocks in every block row (dense blocks, about one nonzero per block between them): mixed dispatch per block
         A = gen.pruned_plus_er(8192, 0.10, 0.001)
         N, bdist, bseed = 4096, "normal", 0xB0000007
+    elif name == "block_pruned_skewed_8192_N4096":
+        # a weight whose rows were pruned unevenly (18 % of the blocks kept in the first block row, 2 % in the last): the
+        # sweep kernel's plan deals the block rows to its row groups by their block count
+        A = gen.block_pruned_skewed(8192, 0.18, 0.02)
+        N, bdist, bseed = 4096, "normal", 0xB0000008
     elif name == "band_4096_bw64_N128":
         d = gen.band(4096, 64)
         b = smat_amd.csr_to_bcsr(d["M"], d["K"], d["row_ptr"], d["col_idx"], d["val"])

@@ -21,7 +21,7 @@ sys.path.insert(0, os.path.dirname(os.path.dirname(HERE)))
 import bench  # noqa: E402
 
 WORKLOADS = ["band_4096_bw64_N128", "er_16384_0.1pct_N256", "er_16384_0.1pct_reordered_N256", "rmat_s20_deg16_N128",
-             "rmat_s20_deg16_reordered_N128", "block_pruned_8192_10pct_N4096", "half_pruned_half_er_8192_N4096", "pruned_plus_er_8192_N4096",
+             "rmat_s20_deg16_reordered_N128", "block_pruned_8192_10pct_N4096", "half_pruned_half_er_8192_N4096", "pruned_plus_er_8192_N4096", "block_pruned_skewed_8192_N4096",
              "stencil27_64_N64", "stencil27_64_reordered_N64", "rmat_s15_deg16_reordered_N128", "rmat_s16_deg16_reordered_N128",
              "rmat_s17_deg16_reordered_N128"]
 OUT = os.path.join(HERE, "structure_hashes.json")
